@@ -1,0 +1,109 @@
+/*
+ * libmxfp8_hip -- MXFP8 (e4m3 + UE8M0 per-32) linear path for AMD MI355X (gfx950).
+ *
+ * C ABI.  Every entry point
+ *   - takes raw DEVICE pointers, sizes and strides; never allocates, frees or
+ *     synchronises; launches on the stream the caller passes (a hipStream_t
+ *     travelling as void*; NULL = the default stream);
+ *   - returns MX_OK or a negative MX_E* code and never throws;
+ *   - is re-entrant: there is no mutable global state.
+ *
+ * The reference (KohakUwULLM) has no FFI; each function cites the reference
+ * Python/Triton interface it stands in for (paths relative to the reference tree).
+ *
+ * Formats.  Codes are OCP float8_e4m3fn bytes.  A scale byte b means 2^(b-127).
+ * A "row-quantized" matrix (R,K) has 32-element blocks along K: codes (R,K) and
+ * scales (R,K/32), both K-minor ("natural" layout of quantize.py:106-137).
+ */
+#ifndef MXFP8_HIP_H
+#define MXFP8_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MX_ABI_VERSION 1
+
+enum mx_status {
+    MX_OK = 0,
+    MX_EINVAL = -1,      /* a size/stride/alignment contract is violated (ValueError upstream) */
+    MX_EUNSUPPORTED = -2, /* well-formed request this build has no kernel for */
+    MX_ELAUNCH = -3,     /* the HIP runtime refused the launch */
+    MX_ENODEV = -4       /* the current device is not gfx950 */
+};
+
+enum mx_dtype { MX_BF16 = 0, MX_FP16 = 1, MX_FP32 = 2 };
+
+/* Epilogues of the GEMM entry points. */
+enum mx_epilogue {
+    MX_EPI_NONE = 0 /* C = A B^T, cast to c_dtype */
+};
+
+int mx_abi_version(void);
+const char *mx_strerror(int status);
+/* 0 when device `dev` is a gfx950 part this library's kernels can run on. */
+int mx_device_supported(int dev);
+
+/*
+ * Row-axis quantizer.  x (M,K) with element strides (sx_row, sx_col) -> q (M,K)
+ * e4m3 with row pitch ldq, s (M,K/32) UE8M0 with row pitch lds.  K % 32 == 0.
+ * Per block: amax in fp32, e = ceil(log2(max(amax,1e-30)/448)), code =
+ * rtne_sat(x / 2^e), byte = e + 127.
+ * Replaces quantize_mx / _quantize_mx_kernel / _quantize_block
+ * (src/kohakuwullm/kernels/mxfp8/quantize.py:39-56,65-137).  A singly-strided
+ * (transposed) input is taken without a copy, as quantize_mx_vendor does
+ * (quantize.py:190-193).
+ */
+int mx_quantize_rows(const void *x, int x_dtype, int64_t M, int64_t K, int64_t sx_row, int64_t sx_col,
+                     uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream);
+
+/*
+ * Column-axis quantizer.  x (M,K) row-major with row pitch ldx -> qT (K,M), sT
+ * (K,M/32): 32-element blocks run along M, outputs are laid out as the row
+ * quantizer's outputs for x^T.  M % 32 == 0.
+ * Replaces quantize_mx(x.t().contiguous()) / quantize_mx_vendor(pad(W.t()))
+ * (src/kohakuwullm/kernels/mxfp8/linear.py:111, moe.py:58-61) without the
+ * transposed copy.
+ */
+int mx_quantize_cols(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                     uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
+
+/*
+ * Both at once, reading x a single time: (q,s) as mx_quantize_rows and (qT,sT)
+ * as mx_quantize_cols.  M % 32 == 0 and K % 32 == 0.
+ * Replaces the pair of quantize calls an activation needs when it feeds both a
+ * forward/dgrad GEMM (blocks along its K) and a wgrad GEMM (blocks along tokens).
+ */
+int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                     uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
+                     uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
+
+/*
+ * q,s = quantize_rows(silu(gate) * up) with the product kept in fp32.
+ * gate, up (M,K) unit inner stride, row pitches ldg, ldu.  K % 32 == 0.
+ * Replaces swiglu_mx / _swiglu_mx_kernel (src/kohakuwullm/kernels/mxfp8/fused_act.py:17-101).
+ */
+int mx_swiglu_quantize_rows(const void *gate, const void *up, int dtype, int64_t M, int64_t K, int64_t ldg,
+                            int64_t ldu, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream);
+
+/*
+ * C (M,N) = deq(A) deq(B)^T, fp32 accumulate, cast to c_dtype (round to nearest
+ * even).  A: codes (M,K) pitch lda + scales (M,K/32) pitch ldas; B: codes (N,K)
+ * pitch ldb + scales (N,K/32) pitch ldbs; both K-minor.  K % 32 == 0.
+ * One entry serves forward (X W^T), dgrad (dY (W^T)^T) and wgrad (dY^T (X^T)^T)
+ * because the quantizers deliver every operand K-minor.
+ * Replaces mxfp8_matmul_pq / _mxfp8_matmul_pq
+ * (src/kohakuwullm/kernels/mxfp8/quantize.py:242-371) and the cuBLAS route
+ * mxfp8_mm_swizzled (src/kohakuwullm/kernels/mxfp8/interop.py:51-122).
+ */
+int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs,
+               void *c, int c_dtype, int64_t M, int64_t N, int64_t K,
+               int64_t lda, int64_t ldas, int64_t ldb, int64_t ldbs, int64_t ldc,
+               int epilogue, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXFP8_HIP_H */

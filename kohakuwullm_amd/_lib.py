@@ -1,0 +1,81 @@
+"""ctypes binding of ``libmxfp8_hip.so`` -- the only door from Python to the HIP kernels.
+
+The library is built in-tree by ``csrc/Makefile`` (``__graft_entry__.build()``).  It is
+loaded after ``import torch`` so that its ``libamdhip64.so.7`` dependency resolves to the
+HIP runtime PyTorch already mapped, which makes PyTorch's streams and device pointers
+valid inside the library.  A missing library or a non-zero status raises: nothing falls
+back to another implementation.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmxfp8_hip.so")
+
+MX_OK, MX_EINVAL, MX_EUNSUPPORTED, MX_ELAUNCH, MX_ENODEV = 0, -1, -2, -3, -4
+MX_DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+_i64, _p, _ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+
+# name -> (restype, argtypes); mirrors include/mxfp8_hip.h declaration by declaration.
+SIGNATURES = {
+    "mx_abi_version": (_ci, []),
+    "mx_strerror": (ctypes.c_char_p, [_ci]),
+    "mx_device_supported": (_ci, [_ci]),
+    "mx_quantize_rows": (_ci, [_p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_quantize_cols": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_swiglu_quantize_rows": (_ci, [_p, _p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),
+}
+
+_lib: ctypes.CDLL | None = None
+
+
+class MXFP8LibraryError(RuntimeError):
+    """The HIP library is missing, or one of its entry points returned an error."""
+
+
+def load() -> ctypes.CDLL:
+    """Load (once) and type the library.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MXFP8LibraryError(
+            f"{LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+            "(or `python -c 'import __graft_entry__ as g; g.build()'`); there is no fallback path"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here means the header and the build disagree
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status == MX_OK:
+        return
+    msg = load().mx_strerror(status).decode()
+    if status == MX_EINVAL:
+        raise ValueError(f"{what}: {msg}")
+    raise MXFP8LibraryError(f"{what}: {msg} (status {status})")
+
+
+def stream_of(t: torch.Tensor) -> int:
+    """The raw hipStream_t PyTorch is currently issuing on for ``t``'s device."""
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise MXFP8LibraryError(
+            f"{name} lives on {t.device}: the MXFP8 kernels run on an MI355X (gfx950) only and have no CPU path"
+        )

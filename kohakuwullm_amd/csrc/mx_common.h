@@ -1,0 +1,117 @@
+// Shared device helpers for the MXFP8 kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mxfp8_hip.h"
+
+#define MX_BLOCK 32
+
+namespace mx {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short v8us __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float bits2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// UE8M0 byte of a block from its fp32 amax (>= 0):
+// ceil(log2(max(amax,1e-30)/448)) + 127 == E - 8 + (M > 0x600000) because 448 = 1.75 * 2^8.
+// quantize.py:53-56 of the reference.
+__device__ __forceinline__ uint32_t scale_byte(float amax) {
+    uint32_t u = f2bits(amax);
+    u = u > 0x0DA24260u ? u : 0x0DA24260u;  // max(amax, 1e-30f) on the bit pattern (amax >= 0)
+    uint32_t e = u >> 23;
+    uint32_t m = u & 0x7FFFFFu;
+    return e - 8u + (m > 0x600000u ? 1u : 0u);
+}
+
+// 2^(127 - byte): multiplying by it divides by the block scale exactly.
+__device__ __forceinline__ float inv_scale(uint32_t byte) { return bits2f((254u - byte) << 23); }
+
+// Two fp32 -> two e4m3 bytes (RTNE) into the low or high half of `old`.
+template <bool HI>
+__device__ __forceinline__ int cvt_pk_e4m3(float a, float b, int old) {
+    return __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, HI);
+}
+
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+    int v = 0;
+    v = cvt_pk_e4m3<false>(a, b, v);
+    v = cvt_pk_e4m3<true>(c, d, v);
+    return (uint32_t)v;
+}
+
+// Element loaders: 8 consecutive elements starting at p (16-byte aligned for 16-bit types).
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<MX_BF16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ void load8(const void *p, float v[8]) {
+        v4i r = *(const v4i *)p;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = bits2f((uint32_t)r[i] << 16);
+            v[2 * i + 1] = bits2f((uint32_t)r[i] & 0xFFFF0000u);
+        }
+    }
+    static __device__ __forceinline__ float load1(const void *p) { return bits2f((uint32_t)(*(const uint16_t *)p) << 16); }
+};
+
+template <>
+struct Elem<MX_FP16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ void load8(const void *p, float v[8]) {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        h8 r = *(const h8 *)p;
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (float)r[i];
+    }
+    static __device__ __forceinline__ float load1(const void *p) { return (float)(*(const _Float16 *)p); }
+};
+
+template <>
+struct Elem<MX_FP32> {
+    typedef float type;
+    static __device__ __forceinline__ void load8(const void *p, float v[8]) {
+        v4f a = ((const v4f *)p)[0], b = ((const v4f *)p)[1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[i] = a[i];
+            v[4 + i] = b[i];
+        }
+    }
+    static __device__ __forceinline__ float load1(const void *p) { return *(const float *)p; }
+};
+
+__device__ __forceinline__ float amax8(const float v[8]) {
+    float a = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fabsf(v[2]));
+    float b = fmaxf(fmaxf(fabsf(v[3]), fabsf(v[4])), fabsf(v[5]));
+    return fmaxf(fmaxf(a, b), fmaxf(fabsf(v[6]), fabsf(v[7])));
+}
+
+// max over the 4 lanes of a quad (DPP quad_perm butterflies); all four lanes get the result.
+__device__ __forceinline__ float quad_max(float a) {
+    int x = __builtin_amdgcn_mov_dpp((int)f2bits(a), 0xB1, 0xF, 0xF, true);  // lane ^ 1
+    a = fmaxf(a, bits2f((uint32_t)x));
+    x = __builtin_amdgcn_mov_dpp((int)f2bits(a), 0x4E, 0xF, 0xF, true);  // lane ^ 2
+    return fmaxf(a, bits2f((uint32_t)x));
+}
+
+// fp32 -> bf16 bits, round to nearest even (finite inputs; NaN keeps a quiet payload).
+__device__ __forceinline__ uint32_t f2bf16(float f) {
+    uint32_t u = f2bits(f);
+    uint32_t r = u + 0x7FFFu + ((u >> 16) & 1u);
+    r = (u & 0x7FFFFFFFu) > 0x7F800000u ? (u | 0x00400000u) : r;
+    return r >> 16;
+}
+
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) { return f2bf16(lo) | (f2bf16(hi) << 16); }
+
+}  // namespace mx

@@ -1,0 +1,436 @@
+// MXFP8 quantizers for gfx950: row axis, column axis, both at once, and SwiGLU -> MXFP8.
+//
+// All of them are HBM-streaming kernels: 16-byte coalesced loads, per-32 amax by a
+// DPP quad reduction (row axis) or an in-register + cross-lane reduction (column
+// axis), the UE8M0 byte from the fp32 exponent/mantissa bits, an exact multiply by
+// 2^-e, and the hardware RTNE e4m3 conversion.  Semantics follow _quantize_block of
+// the reference (src/kohakuwullm/kernels/mxfp8/quantize.py:39-56).
+#include "mx_common.h"
+
+namespace mx {
+
+// ------------------------------------------------------------------------------------
+// Row axis.  One lane owns 8 consecutive elements; the 4 lanes of a quad own one block.
+// ------------------------------------------------------------------------------------
+
+// OR the quad's byte into a dword holding the 4 bytes of a 16-lane row, in block order.
+__device__ __forceinline__ uint32_t gather_row_scales(uint32_t byte, int lane) {
+    uint32_t v = byte << ((lane & 12) << 1);
+    v |= (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x124, 0xF, 0xF, true);  // row_ror:4
+    v |= (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x128, 0xF, 0xF, true);  // row_ror:8
+    return v;
+}
+
+template <int DT, int U, bool FLAT>
+__global__ __launch_bounds__(256) void quant_rows_kernel(const void *__restrict__ x, uint32_t chunks_per_row,
+                                                          int64_t sx_row, uint8_t *__restrict__ q, int64_t ldq,
+                                                          uint8_t *__restrict__ s, int64_t lds, uint32_t total_chunks,
+                                                          int pack_scales) {
+    typedef typename Elem<DT>::type T;
+    const int lane = threadIdx.x & 63;
+    const uint32_t base = blockIdx.x * (uint32_t)(U * 256) + threadIdx.x;
+    float v[U][8];
+    int64_t qoff[U], soff[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        uint32_t chunk = base + u * 256;
+        ok[u] = chunk < total_chunks;
+        int64_t xoff;
+        if (FLAT) {
+            xoff = (int64_t)chunk * 8;
+            qoff[u] = (int64_t)chunk * 8;
+            soff[u] = chunk >> 2;
+        } else {
+            uint32_t row = chunk / chunks_per_row;
+            uint32_t col = chunk - row * chunks_per_row;
+            xoff = (int64_t)row * sx_row + (int64_t)col * 8;
+            qoff[u] = (int64_t)row * ldq + (int64_t)col * 8;
+            soff[u] = (int64_t)row * lds + (col >> 2);
+        }
+        if (ok[u]) {
+            Elem<DT>::load8((const T *)x + xoff, v[u]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[u][i] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float amax = quad_max(amax8(v[u]));
+        uint32_t byte = scale_byte(amax);
+        float inv = inv_scale(byte);
+        uint32_t packed = gather_row_scales(byte, lane);
+        if (ok[u]) {
+            v2i codes;
+            codes[0] = (int)pack4_e4m3(v[u][0] * inv, v[u][1] * inv, v[u][2] * inv, v[u][3] * inv);
+            codes[1] = (int)pack4_e4m3(v[u][4] * inv, v[u][5] * inv, v[u][6] * inv, v[u][7] * inv);
+            *(v2i *)(q + qoff[u]) = codes;
+            // The 16 lanes of a DPP row hold 4 consecutive blocks.  They are all valid or
+            // the tail of the tensor cuts the group, in which case bytes are stored singly.
+            bool group_full = ((base + u * 256) | 15u) < total_chunks;
+            if (pack_scales && group_full) {
+                if ((lane & 15) == 0) *(uint32_t *)(s + soff[u]) = packed;
+            } else if ((lane & 3) == 0) {
+                s[soff[u]] = (uint8_t)byte;
+            }
+        }
+    }
+}
+
+// Any strides: one thread per block.  The slow path for doubly-strided views.
+template <int DT>
+__global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__restrict__ x, int64_t M, int64_t KB,
+                                                                  int64_t sx_row, int64_t sx_col,
+                                                                  uint8_t *__restrict__ q, int64_t ldq,
+                                                                  uint8_t *__restrict__ s, int64_t lds) {
+    typedef typename Elem<DT>::type T;
+    int64_t blk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (blk >= M * KB) return;
+    int64_t row = blk / KB, kb = blk - row * KB;
+    const T *p = (const T *)x + row * sx_row + kb * MX_BLOCK * sx_col;
+    float v[MX_BLOCK];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MX_BLOCK; i++) {
+        v[i] = Elem<DT>::load1(p + i * sx_col);
+        amax = fmaxf(amax, fabsf(v[i]));
+    }
+    uint32_t byte = scale_byte(amax);
+    float inv = inv_scale(byte);
+    uint8_t *qo = q + row * ldq + kb * MX_BLOCK;
+#pragma unroll
+    for (int i = 0; i < MX_BLOCK; i += 4) {
+        uint32_t c = pack4_e4m3(v[i] * inv, v[i + 1] * inv, v[i + 2] * inv, v[i + 3] * inv);
+        qo[i] = (uint8_t)c;
+        qo[i + 1] = (uint8_t)(c >> 8);
+        qo[i + 2] = (uint8_t)(c >> 16);
+        qo[i + 3] = (uint8_t)(c >> 24);
+    }
+    s[row * lds + kb] = (uint8_t)byte;
+}
+
+// ------------------------------------------------------------------------------------
+// Column axis (and dual).  A 256-thread workgroup owns a 128 (M) x 128 (K) tile.  Thread
+// (cg = t%16, rg = t/16) holds rows rg*8..+7 x columns cg*8..+7, so wave w holds exactly
+// the w-th 32-row block of the tile: the column amax is an in-register max over 8 rows
+// and a max across the wave's 4 row groups (lanes l, l^16, l^32, l^48).  Codes are
+// transposed through LDS so the (K,M) output is written in full 128-byte rows.
+// ------------------------------------------------------------------------------------
+
+#define QC_TILE 128
+#define QC_PITCH 136  // bytes per transposed LDS row (8-byte aligned, staggers banks)
+
+template <int DT, bool DUAL>
+__global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict__ x, int64_t M, int64_t K, int64_t ldx,
+                                                          uint8_t *__restrict__ qT, int64_t ldqT,
+                                                          uint8_t *__restrict__ sT, int64_t ldsT,
+                                                          uint8_t *__restrict__ q, int64_t ldq,
+                                                          uint8_t *__restrict__ s, int64_t lds, int pack_row_scales,
+                                                          int pack_col_scales) {
+    typedef typename Elem<DT>::type T;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int cg = t & 15, rg = t >> 4;
+    const int64_t m0 = (int64_t)blockIdx.y * QC_TILE, k0 = (int64_t)blockIdx.x * QC_TILE;
+    const int64_t col = k0 + cg * 8;
+    const int64_t row0 = m0 + rg * 8;
+    const bool col_ok = col < K;                     // K % 8 == 0: an 8-column chunk is in or out
+    const bool blk_ok = m0 + wave * 32 < M;          // M % 32 == 0: a 32-row block is in or out
+
+    float v[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (col_ok && blk_ok) {
+            Elem<DT>::load8((const T *)x + (row0 + i) * ldx + col, v[i]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
+        }
+    }
+
+    if (DUAL) {
+        // Row-axis outputs: the 4 lanes of a quad hold 32 consecutive columns of a row.
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float amax = quad_max(amax8(v[i]));
+            uint32_t byte = scale_byte(amax);
+            float inv = inv_scale(byte);
+            uint32_t packed = gather_row_scales(byte, lane);
+            if (col_ok && blk_ok) {
+                v2i codes;
+                codes[0] = (int)pack4_e4m3(v[i][0] * inv, v[i][1] * inv, v[i][2] * inv, v[i][3] * inv);
+                codes[1] = (int)pack4_e4m3(v[i][4] * inv, v[i][5] * inv, v[i][6] * inv, v[i][7] * inv);
+                *(v2i *)(q + (row0 + i) * ldq + col) = codes;
+                uint8_t *sp = s + (row0 + i) * lds + (col >> 5);
+                bool full = k0 + QC_TILE <= K;
+                if (pack_row_scales && full) {
+                    if (cg == 0) *(uint32_t *)sp = packed;
+                } else if ((cg & 3) == 0) {
+                    *sp = (uint8_t)byte;
+                }
+            }
+        }
+    }
+
+    // Column amax over this wave's 32 rows.
+    float cm[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        float a = fmaxf(fmaxf(fabsf(v[0][c]), fabsf(v[1][c])), fabsf(v[2][c]));
+        float b = fmaxf(fmaxf(fabsf(v[3][c]), fabsf(v[4][c])), fabsf(v[5][c]));
+        cm[c] = fmaxf(fmaxf(a, b), fmaxf(fabsf(v[6][c]), fabsf(v[7][c])));
+    }
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        cm[c] = fmaxf(cm[c], __shfl_xor(cm[c], 16, 64));
+        cm[c] = fmaxf(cm[c], __shfl_xor(cm[c], 32, 64));
+    }
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        uint32_t byte = scale_byte(cm[c]);
+        float inv = inv_scale(byte);
+        v2i codes;
+        codes[0] = (int)pack4_e4m3(v[0][c] * inv, v[1][c] * inv, v[2][c] * inv, v[3][c] * inv);
+        codes[1] = (int)pack4_e4m3(v[4][c] * inv, v[5][c] * inv, v[6][c] * inv, v[7][c] * inv);
+        *(v2i *)(tile + (cg * 8 + c) * QC_PITCH + rg * 8) = codes;
+        if ((rg & 3) == 0) tscale[(cg * 8 + c) * 4 + wave] = (uint8_t)byte;
+    }
+    __syncthreads();
+
+    // Transposed codes: 128 rows of 128 bytes, 16 bytes per thread per pass.
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int kr = j * 32 + (t >> 3), ch = t & 7;
+        if (k0 + kr < K && m0 + ch * 16 < M) {
+            const v2i *src = (const v2i *)(tile + kr * QC_PITCH + ch * 16);
+            v4i o;
+            v2i a = src[0], b = src[1];
+            o[0] = a[0];
+            o[1] = a[1];
+            o[2] = b[0];
+            o[3] = b[1];
+            *(v4i *)(qT + (k0 + kr) * ldqT + m0 + ch * 16) = o;
+        }
+    }
+    if (t < QC_TILE && k0 + t < K) {
+        uint8_t *sp = sT + (k0 + t) * ldsT + (m0 >> 5);
+        int64_t nb = (M - m0) >> 5;
+        if (pack_col_scales && nb >= 4) {
+            *(uint32_t *)sp = *(const uint32_t *)(tscale + t * 4);
+        } else {
+            for (int b = 0; b < 4 && b < nb; b++) sp[b] = tscale[t * 4 + b];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// silu(gate) * up in fp32 -> row-axis MXFP8 (fused_act.py:37-66 of the reference).
+// ------------------------------------------------------------------------------------
+
+template <int DT, int U>
+__global__ __launch_bounds__(256) void swiglu_quant_rows_kernel(const void *__restrict__ g, const void *__restrict__ up,
+                                                                 uint32_t chunks_per_row, int64_t ldg, int64_t ldu,
+                                                                 uint8_t *__restrict__ q, int64_t ldq,
+                                                                 uint8_t *__restrict__ s, int64_t lds,
+                                                                 uint32_t total_chunks, int pack_scales) {
+    typedef typename Elem<DT>::type T;
+    const int lane = threadIdx.x & 63;
+    const uint32_t base = blockIdx.x * (uint32_t)(U * 256) + threadIdx.x;
+    float a[U][8], b[U][8];
+    int64_t qoff[U], soff[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        uint32_t chunk = base + u * 256;
+        ok[u] = chunk < total_chunks;
+        uint32_t row = chunk / chunks_per_row;
+        uint32_t col = chunk - row * chunks_per_row;
+        qoff[u] = (int64_t)row * ldq + (int64_t)col * 8;
+        soff[u] = (int64_t)row * lds + (col >> 2);
+        if (ok[u]) {
+            Elem<DT>::load8((const T *)g + (int64_t)row * ldg + (int64_t)col * 8, a[u]);
+            Elem<DT>::load8((const T *)up + (int64_t)row * ldu + (int64_t)col * 8, b[u]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) a[u][i] = b[u][i] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float gv = a[u][i];
+            v[i] = gv * __fdividef(1.0f, 1.0f + __expf(-gv)) * b[u][i];
+        }
+        float amax = quad_max(amax8(v));
+        uint32_t byte = scale_byte(amax);
+        float inv = inv_scale(byte);
+        uint32_t packed = gather_row_scales(byte, lane);
+        if (ok[u]) {
+            v2i codes;
+            codes[0] = (int)pack4_e4m3(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+            codes[1] = (int)pack4_e4m3(v[4] * inv, v[5] * inv, v[6] * inv, v[7] * inv);
+            *(v2i *)(q + qoff[u]) = codes;
+            bool group_full = ((base + u * 256) | 15u) < total_chunks;
+            if (pack_scales && group_full) {
+                if ((lane & 15) == 0) *(uint32_t *)(s + soff[u]) = packed;
+            } else if ((lane & 3) == 0) {
+                s[soff[u]] = (uint8_t)byte;
+            }
+        }
+    }
+}
+
+}  // namespace mx
+
+// ------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------
+
+using namespace mx;
+
+static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+static inline int esize(int dt) { return dt == MX_FP32 ? 4 : 2; }
+
+#define MX_LAUNCH_CHECK()                                   \
+    do {                                                    \
+        if (hipGetLastError() != hipSuccess) return MX_ELAUNCH; \
+    } while (0)
+
+template <int DT>
+static int launch_rows(const void *x, int64_t M, int64_t K, int64_t sx_row, int64_t sx_col, uint8_t *q, int64_t ldq,
+                       uint8_t *s, int64_t lds, hipStream_t st) {
+    const int64_t KB = K / MX_BLOCK;
+    const bool vec_ok = sx_col == 1 && aligned(x, 16) && (sx_row * esize(DT)) % 16 == 0 && aligned(q, 8) &&
+                        ldq % 8 == 0 && M * (K / 8) < (int64_t)0x7FFFFF00;
+    if (!vec_ok) {
+        int64_t blocks = M * KB;
+        if ((blocks + 255) / 256 > 0x7FFFFFFF) return MX_EUNSUPPORTED;
+        quant_rows_generic_kernel<DT><<<dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, st>>>(
+            x, M, KB, sx_row, sx_col, q, ldq, s, lds);
+        MX_LAUNCH_CHECK();
+        return MX_OK;
+    }
+    constexpr int U = 4;
+    const uint32_t cpr = (uint32_t)(K / 8);
+    const uint32_t total = (uint32_t)(M * (K / 8));
+    const unsigned grid = (total + U * 256 - 1) / (U * 256);
+    const bool flat = sx_row == K && ldq == K && lds == KB;
+    if (flat) {
+        int pack = aligned(s, 4);
+        quant_rows_kernel<DT, U, true><<<dim3(grid), dim3(256), 0, st>>>(x, cpr, sx_row, q, ldq, s, lds, total, pack);
+    } else {
+        int pack = aligned(s, 4) && lds % 4 == 0 && KB % 4 == 0;
+        quant_rows_kernel<DT, U, false><<<dim3(grid), dim3(256), 0, st>>>(x, cpr, sx_row, q, ldq, s, lds, total, pack);
+    }
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+template <int DT, bool DUAL>
+static int launch_cols(const void *x, int64_t M, int64_t K, int64_t ldx, uint8_t *qT, int64_t ldqT, uint8_t *sT,
+                       int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, hipStream_t st) {
+    dim3 grid((unsigned)((K + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
+    if (grid.y > 65535u) return MX_EUNSUPPORTED;
+    int pack_row = DUAL && aligned(s, 4) && lds % 4 == 0;
+    int pack_col = aligned(sT, 4) && ldsT % 4 == 0;
+    quant_cols_kernel<DT, DUAL><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, pack_row,
+                                                             pack_col);
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+static bool cols_vec_ok(const void *x, int dt, int64_t K, int64_t ldx, const uint8_t *qT, int64_t ldqT) {
+    return K % 8 == 0 && aligned(x, 16) && (ldx * esize(dt)) % 16 == 0 && aligned(qT, 16) && ldqT % 16 == 0;
+}
+
+extern "C" int mx_quantize_cols(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, uint8_t *qT,
+                                int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream) {
+    if (M < 0 || K < 0 || M % MX_BLOCK || ldx < K || ldqT < M || ldsT < M / MX_BLOCK) return MX_EINVAL;
+    if (M == 0 || K == 0) return MX_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (!cols_vec_ok(x, x_dtype, K, ldx, qT, ldqT)) {
+        // Rows of the transposed view, one thread per block.
+        switch (x_dtype) {
+        case MX_BF16: return launch_rows<MX_BF16>(x, K, M, 1, ldx, qT, ldqT, sT, ldsT, st);
+        case MX_FP16: return launch_rows<MX_FP16>(x, K, M, 1, ldx, qT, ldqT, sT, ldsT, st);
+        case MX_FP32: return launch_rows<MX_FP32>(x, K, M, 1, ldx, qT, ldqT, sT, ldsT, st);
+        default: return MX_EINVAL;
+        }
+    }
+    switch (x_dtype) {
+    case MX_BF16: return launch_cols<MX_BF16, false>(x, M, K, ldx, qT, ldqT, sT, ldsT, nullptr, 0, nullptr, 0, st);
+    case MX_FP16: return launch_cols<MX_FP16, false>(x, M, K, ldx, qT, ldqT, sT, ldsT, nullptr, 0, nullptr, 0, st);
+    case MX_FP32: return launch_cols<MX_FP32, false>(x, M, K, ldx, qT, ldqT, sT, ldsT, nullptr, 0, nullptr, 0, st);
+    default: return MX_EINVAL;
+    }
+}
+
+extern "C" int mx_quantize_rows(const void *x, int x_dtype, int64_t M, int64_t K, int64_t sx_row, int64_t sx_col,
+                                uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream) {
+    if (M < 0 || K < 0 || K % MX_BLOCK || ldq < K || lds < K / MX_BLOCK) return MX_EINVAL;
+    if (M == 0 || K == 0) return MX_OK;
+    hipStream_t st = (hipStream_t)stream;
+    // A transposed view (unit stride down the rows) is the column quantizer of the
+    // matrix underneath it: no copy is made.
+    if (sx_col != 1 && sx_row == 1 && M > 1 && cols_vec_ok(x, x_dtype, M, sx_col, q, ldq))
+        return mx_quantize_cols(x, x_dtype, K, M, sx_col, q, ldq, s, lds, stream);
+    switch (x_dtype) {
+    case MX_BF16: return launch_rows<MX_BF16>(x, M, K, sx_row, sx_col, q, ldq, s, lds, st);
+    case MX_FP16: return launch_rows<MX_FP16>(x, M, K, sx_row, sx_col, q, ldq, s, lds, st);
+    case MX_FP32: return launch_rows<MX_FP32>(x, M, K, sx_row, sx_col, q, ldq, s, lds, st);
+    default: return MX_EINVAL;
+    }
+}
+
+extern "C" int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, uint8_t *q, int64_t ldq,
+                                uint8_t *s, int64_t lds, uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT,
+                                void *stream) {
+    if (M < 0 || K < 0 || M % MX_BLOCK || K % MX_BLOCK || ldx < K || ldq < K || lds < K / MX_BLOCK || ldqT < M ||
+        ldsT < M / MX_BLOCK)
+        return MX_EINVAL;
+    if (M == 0 || K == 0) return MX_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (!cols_vec_ok(x, x_dtype, K, ldx, qT, ldqT) || !aligned(q, 8) || ldq % 8) {
+        int rc = mx_quantize_rows(x, x_dtype, M, K, ldx, 1, q, ldq, s, lds, stream);
+        if (rc != MX_OK) return rc;
+        return mx_quantize_cols(x, x_dtype, M, K, ldx, qT, ldqT, sT, ldsT, stream);
+    }
+    switch (x_dtype) {
+    case MX_BF16: return launch_cols<MX_BF16, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
+    case MX_FP16: return launch_cols<MX_FP16, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
+    case MX_FP32: return launch_cols<MX_FP32, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
+    default: return MX_EINVAL;
+    }
+}
+
+template <int DT>
+static int launch_swiglu(const void *g, const void *u, int64_t M, int64_t K, int64_t ldg, int64_t ldu, uint8_t *q,
+                         int64_t ldq, uint8_t *s, int64_t lds, hipStream_t st) {
+    constexpr int U = 2;
+    const uint32_t total = (uint32_t)(M * (K / 8));
+    const unsigned grid = (total + U * 256 - 1) / (U * 256);
+    int pack = aligned(s, 4) && lds % 4 == 0 && (K / MX_BLOCK) % 4 == 0;
+    swiglu_quant_rows_kernel<DT, U><<<dim3(grid), dim3(256), 0, st>>>(g, u, (uint32_t)(K / 8), ldg, ldu, q, ldq, s, lds,
+                                                                      total, pack);
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+extern "C" int mx_swiglu_quantize_rows(const void *gate, const void *up, int dtype, int64_t M, int64_t K, int64_t ldg,
+                                       int64_t ldu, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream) {
+    if (M < 0 || K < 0 || K % MX_BLOCK || ldg < K || ldu < K || ldq < K || lds < K / MX_BLOCK) return MX_EINVAL;
+    if (M == 0 || K == 0) return MX_OK;
+    if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
+    if (!aligned(gate, 16) || !aligned(up, 16) || (ldg * 2) % 16 || (ldu * 2) % 16 || !aligned(q, 8) || ldq % 8 ||
+        M * (K / 8) >= (int64_t)0x7FFFFF00)
+        return MX_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == MX_BF16 ? launch_swiglu<MX_BF16>(gate, up, M, K, ldg, ldu, q, ldq, s, lds, st)
+                            : launch_swiglu<MX_FP16>(gate, up, M, K, ldg, ldu, q, ldq, s, lds, st);
+}

@@ -1,0 +1,42 @@
+"""Activation epilogue that emits MXFP8 directly, so the consumer GEMM needs no cast.
+
+Mirrors ``swiglu_mx`` of the reference (``src/kohakuwullm/kernels/mxfp8/fused_act.py:69-101``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kohakuwullm_amd import _lib
+from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE
+
+
+def swiglu_mx(gate: torch.Tensor, up: torch.Tensor):
+    """``silu(gate) * up`` as ``(e4m3 (M,K), ue8m0 (M, K//32))``; K a multiple of 32.
+
+    The product is kept in fp32 and quantized from there.
+    """
+    if gate.shape != up.shape:
+        raise ValueError(f"gate {tuple(gate.shape)} != up {tuple(up.shape)}")
+    if gate.shape[-1] % BLOCK_SCALE:
+        raise ValueError(f"K={gate.shape[-1]} must be a multiple of {BLOCK_SCALE}")
+    if gate.dtype != up.dtype or gate.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError(f"gate/up must share a 16-bit dtype, got {gate.dtype}, {up.dtype}")
+    _lib.require_gpu(gate, "gate")
+    shape = gate.shape
+    g2, u2 = gate.reshape(-1, shape[-1]), up.reshape(-1, shape[-1])
+    # chunked halves of one projection are accepted through their row pitch
+    if g2.stride(1) != 1:
+        g2 = g2.contiguous()
+    if u2.stride(1) != 1:
+        u2 = u2.contiguous()
+    m, k = g2.shape
+    q = torch.empty(m, k, device=gate.device, dtype=torch.float8_e4m3fn)
+    s = torch.empty(m, k // BLOCK_SCALE, device=gate.device, dtype=torch.uint8)
+    if m and k:
+        rc = _lib.load().mx_swiglu_quantize_rows(
+            g2.data_ptr(), u2.data_ptr(), _lib.MX_DTYPE[gate.dtype], m, k, g2.stride(0), u2.stride(0),
+            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE, _lib.stream_of(gate),
+        )
+        _lib.check(rc, "mx_swiglu_quantize_rows")
+    return q, s

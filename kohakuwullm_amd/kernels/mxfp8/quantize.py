@@ -1,0 +1,166 @@
+"""MXFP8 quantizers and the pre-quantized GEMM, on hand-written gfx950 kernels.
+
+Same names, arguments, return dtypes and errors as the reference module
+``src/kohakuwullm/kernels/mxfp8/quantize.py`` (``quantize_mx`` :106-137,
+``mxfp8_matmul_pq`` :328-371, ``mxfp8_matmul`` :433-473), plus the column-axis and
+dual quantizers the MXFP8 wgrad needs (the reference realises the column axis as
+``quantize_mx(x.t())``: ``linear.py:111``, ``moe.py:58-61``).
+
+Block scales run along the contraction axis and the scale exponent rounds up.
+Accumulation is fp32 always; the output dtype is the caller's.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kohakuwullm_amd import _lib
+
+E4M3_MAX = 448.0
+BLOCK_SCALE = 32
+
+_FP8 = torch.float8_e4m3fn
+
+
+def _check_2d(x: torch.Tensor, name: str) -> None:
+    if x.dim() != 2:
+        raise ValueError(f"{name} must be 2-D, got shape {tuple(x.shape)}")
+    if x.dtype not in _lib.MX_DTYPE:
+        raise ValueError(f"{name}.dtype={x.dtype} is not one of {tuple(_lib.MX_DTYPE)}")
+    _lib.require_gpu(x, name)
+
+
+def quantize_mx(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(M,K)`` -> ``(e4m3 (M,K), ue8m0 (M, K//32))``, blocks along the last axis.
+
+    Bandwidth-bound.  ``K`` must be a multiple of 32.  Any strides are accepted; a
+    transposed view is quantized in place of a copy (the column-axis kernel runs on
+    the matrix underneath it).
+    """
+    if x.shape[-1] % BLOCK_SCALE:
+        raise ValueError(f"K={x.shape[-1]} must be a multiple of {BLOCK_SCALE}")
+    _check_2d(x, "x")
+    m, k = x.shape
+    q = torch.empty(m, k, device=x.device, dtype=_FP8)
+    s = torch.empty(m, k // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+    if m and k:
+        rc = _lib.load().mx_quantize_rows(
+            x.data_ptr(), _lib.MX_DTYPE[x.dtype], m, k, x.stride(0), x.stride(1),
+            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE, _lib.stream_of(x),
+        )
+        _lib.check(rc, "mx_quantize_rows")
+    return q, s
+
+
+def quantize_mx_cols(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(M,K)`` -> ``(e4m3 (K,M), ue8m0 (K, M//32))``: blocks of 32 along ``M``.
+
+    Equal, bit for bit, to ``quantize_mx(x.t().contiguous())`` without the copy.
+    ``M`` must be a multiple of 32.
+    """
+    if x.shape[0] % BLOCK_SCALE:
+        raise ValueError(f"M={x.shape[0]} must be a multiple of {BLOCK_SCALE}")
+    _check_2d(x, "x")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    m, k = x.shape
+    qt = torch.empty(k, m, device=x.device, dtype=_FP8)
+    st = torch.empty(k, m // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+    if m and k:
+        rc = _lib.load().mx_quantize_cols(
+            x.data_ptr(), _lib.MX_DTYPE[x.dtype], m, k, x.stride(0),
+            qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE, _lib.stream_of(x),
+        )
+        _lib.check(rc, "mx_quantize_cols")
+    return qt, st
+
+
+def quantize_mx_dual(x: torch.Tensor):
+    """Row- and column-axis quantization of ``x`` in one pass over it.
+
+    Returns ``(q, s, qT, sT)`` with ``(q, s) == quantize_mx(x)`` and
+    ``(qT, sT) == quantize_mx_cols(x)``.  Both ``M`` and ``K`` must be multiples of 32.
+    """
+    if x.shape[-1] % BLOCK_SCALE or x.shape[0] % BLOCK_SCALE:
+        raise ValueError(f"shape {tuple(x.shape)}: both axes must be multiples of {BLOCK_SCALE}")
+    _check_2d(x, "x")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    m, k = x.shape
+    q = torch.empty(m, k, device=x.device, dtype=_FP8)
+    s = torch.empty(m, k // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+    qt = torch.empty(k, m, device=x.device, dtype=_FP8)
+    st = torch.empty(k, m // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+    if m and k:
+        rc = _lib.load().mx_quantize_dual(
+            x.data_ptr(), _lib.MX_DTYPE[x.dtype], m, k, x.stride(0),
+            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE,
+            qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE, _lib.stream_of(x),
+        )
+        _lib.check(rc, "mx_quantize_dual")
+    return q, s, qt, st
+
+
+def _gemm_nt_into(aq, a_scale, bq, b_scale, out) -> None:
+    m, k = aq.shape
+    n = bq.shape[0]
+    rc = _lib.load().mx_gemm_nt(
+        aq.data_ptr(), a_scale.data_ptr(), bq.data_ptr(), b_scale.data_ptr(), out.data_ptr(),
+        _lib.MX_DTYPE[out.dtype], m, n, k, aq.stride(0), a_scale.stride(0), bq.stride(0), b_scale.stride(0),
+        out.stride(0), 0, _lib.stream_of(aq),
+    )
+    _lib.check(rc, "mx_gemm_nt")
+
+
+def mxfp8_matmul_pq(
+    aq: torch.Tensor,
+    a_scale: torch.Tensor,
+    bq: torch.Tensor,
+    b_scale: torch.Tensor,
+    out_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """``aq @ bq.T`` from pre-quantized operands, fp32 accumulate.
+
+    ``aq (M,K)``, ``bq (N,K)`` e4m3 and ``a_scale (M,K//32)``, ``b_scale (N,K//32)``
+    ue8m0 in the natural layout ``quantize_mx`` produces.  Needs only ``K % 32 == 0``.
+    """
+    if aq.dim() != 2 or bq.dim() != 2 or aq.shape[1] != bq.shape[1]:
+        raise ValueError(f"contraction mismatch: {tuple(aq.shape)} @ {tuple(bq.shape)}.T")
+    m, k = aq.shape
+    n = bq.shape[0]
+    if k % BLOCK_SCALE:
+        raise ValueError(f"K={k} must be a multiple of {BLOCK_SCALE}")
+    if a_scale.shape != (m, k // BLOCK_SCALE) or b_scale.shape != (n, k // BLOCK_SCALE):
+        raise ValueError(
+            f"scale shapes {tuple(a_scale.shape)}, {tuple(b_scale.shape)} do not match operands "
+            f"{tuple(aq.shape)}, {tuple(bq.shape)}"
+        )
+    if out_dtype not in _lib.MX_DTYPE:
+        raise ValueError(f"out_dtype={out_dtype} is not one of {tuple(_lib.MX_DTYPE)}")
+    _lib.require_gpu(aq, "aq")
+    tensors = []
+    for t in (aq, a_scale, bq, b_scale):
+        if t.element_size() != 1:
+            raise ValueError(f"codes and scales must be 1-byte tensors, got {t.dtype}")
+        tensors.append(t if t.stride(1) == 1 else t.contiguous())
+    out = torch.empty(m, n, device=aq.device, dtype=out_dtype)
+    if m and n:
+        _gemm_nt_into(*tensors, out)
+    return out
+
+
+def mxfp8_matmul(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``a @ b.T`` in MXFP8 with fp32 accumulation: quantize both, then multiply.
+
+    Args:
+        a: ``(M, K)`` activations in fp16/bf16.
+        b: ``(N, K)`` weights in fp16/bf16, K-minor as a linear layer stores them.
+        out_dtype: output dtype; defaults to ``a``'s.
+    """
+    if a.shape[-1] != b.shape[-1]:
+        raise ValueError(f"contraction mismatch: {a.shape} @ {b.shape}.T")
+    if a.shape[-1] % BLOCK_SCALE:
+        raise ValueError(f"K={a.shape[-1]} must be a multiple of {BLOCK_SCALE}")
+    aq, a_scale = quantize_mx(a)
+    bq, b_scale = quantize_mx(b)
+    return mxfp8_matmul_pq(aq, a_scale, bq, b_scale, out_dtype or a.dtype)

@@ -1,0 +1,191 @@
+"""Parity of the HIP quantizers with the CPU oracle: bit-exact codes and scales.
+
+Calls go through the C ABI (ctypes -> libmxfp8_hip.so).  Inputs are drawn on a CPU
+generator and copied to the device so both sides see the same bits.
+"""
+
+import pytest
+import torch
+
+from conftest import SEED
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _mx():
+    from kohakuwullm_amd.kernels import mxfp8
+
+    return mxfp8
+
+
+def _rand(shape, dtype, scale=1.0, seed=SEED):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def _eq(got, ref, what):
+    got = got.view(torch.uint8).cpu()
+    if not torch.equal(got, ref):
+        bad = (got != ref).nonzero()
+        raise AssertionError(f"{what}: {bad.shape[0]} mismatches, first at {bad[0].tolist()}: got {got[tuple(bad[0])]} ref {ref[tuple(bad[0])]}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 32), (3, 96), (8, 1024), (257, 160), (96, 4096), (1000, 512)])
+def test_rows_bit_exact(oracle, dtype, shape):
+    x = _rand(shape, dtype, 1.0)
+    q, s = _mx().quantize_mx(x.to(DEV))
+    qr, sr = oracle.quantize_rows(x)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.uint8
+    _eq(s, sr, "scales")
+    _eq(q, qr, "codes")
+
+
+@pytest.mark.parametrize("scale", [0.02, 1e-2, 1e-2 * 2.0**-20, 300.0, 1e30])
+def test_rows_scales_of_magnitude(oracle, scale):
+    x = _rand((64, 512), torch.bfloat16, scale)
+    q, s = _mx().quantize_mx(x.to(DEV))
+    qr, sr = oracle.quantize_rows(x)
+    _eq(s, sr, "scales")
+    _eq(q, qr, "codes")
+
+
+def test_rows_every_bf16_value(oracle):
+    """Each finite bf16 value as the amax of a block, with every other finite bf16 value beside it."""
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = bits[torch.isfinite(bits.float())]
+    n = finite.numel()  # 65280
+    g = torch.Generator().manual_seed(SEED)
+    # block = [amax candidate, 31 random finite values]; 2040 rows x 32 blocks
+    x = finite[torch.randint(0, n, (n, 32), generator=g)]
+    x[:, 0] = finite
+    x = x.reshape(-1, 1024).contiguous()
+    q, s = _mx().quantize_mx(x.to(DEV))
+    qr, sr = oracle.quantize_rows(x)
+    _eq(s, sr, "scales")
+    _eq(q, qr, "codes")
+
+
+def test_rows_edge_blocks(oracle):
+    x = _rand((16, 256), torch.bfloat16)
+    x[0, :32] = 0.0
+    x[1, 32:64] = 1e-35
+    x[2, 64] = 3.0e38
+    x[2, 65] = -3.0e38
+    x[3, :32] = 0.0
+    x[3, 5] = -448.0 * 8
+    x[4, 96:128] = -0.0
+    x[5, 128:160] = 2.0**-133  # bf16 subnormal
+    q, s = _mx().quantize_mx(x.to(DEV))
+    qr, sr = oracle.quantize_rows(x)
+    _eq(s, sr, "scales")
+    _eq(q, qr, "codes")
+    assert s[0, 0] == 19 and s[2, 2] == 247 and s[3, 0] == 130
+
+
+def test_rows_strided_views(oracle):
+    base = _rand((320, 384), torch.bfloat16, 2.0)
+    dev = base.to(DEV)
+    # row-pitch view
+    q, s = _mx().quantize_mx(dev[:, 64:320])
+    qr, sr = oracle.quantize_rows(base[:, 64:320])
+    _eq(s, sr, "pitch scales")
+    _eq(q, qr, "pitch codes")
+    # transposed view: no copy, column kernel underneath
+    q, s = _mx().quantize_mx(dev.t())
+    qr, sr = oracle.quantize_rows(base.t())
+    _eq(s, sr, "transposed scales")
+    _eq(q, qr, "transposed codes")
+    # doubly strided view: generic kernel
+    q, s = _mx().quantize_mx(dev[::2, ::2][:, :160])
+    qr, sr = oracle.quantize_rows(base[::2, ::2][:, :160])
+    _eq(s, sr, "generic scales")
+    _eq(q, qr, "generic codes")
+
+
+def test_rows_errors():
+    mx = _mx()
+    with pytest.raises(ValueError):
+        mx.quantize_mx(torch.zeros(4, 48, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(ValueError):
+        mx.quantize_mx_cols(torch.zeros(48, 64, dtype=torch.bfloat16, device=DEV))
+    q, s = mx.quantize_mx(torch.zeros(0, 64, dtype=torch.bfloat16, device=DEV))
+    assert q.shape == (0, 64) and s.shape == (0, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(32, 8), (64, 128), (160, 136), (128, 1000), (1024, 384), (96, 2048)])
+def test_cols_bit_exact(oracle, dtype, shape):
+    x = _rand(shape, dtype, 1.5)
+    qt, st = _mx().quantize_mx_cols(x.to(DEV))
+    qr, sr = oracle.quantize_cols(x)
+    assert qt.shape == (shape[1], shape[0]) and st.shape == (shape[1], shape[0] // 32)
+    _eq(st, sr, "scales")
+    _eq(qt, qr, "codes")
+
+
+def test_cols_unaligned_falls_back(oracle):
+    x = _rand((64, 100), torch.bfloat16)  # K % 8 != 0 -> generic path
+    qt, st = _mx().quantize_mx_cols(x.to(DEV))
+    qr, sr = oracle.quantize_cols(x)
+    _eq(st, sr, "scales")
+    _eq(qt, qr, "codes")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(32, 32), (128, 128), (160, 96), (512, 1536), (96, 4096)])
+def test_dual_bit_exact(oracle, dtype, shape):
+    x = _rand(shape, dtype, 0.7)
+    q, s, qt, st = _mx().quantize_mx_dual(x.to(DEV))
+    qr, sr = oracle.quantize_rows(x)
+    qtr, str_ = oracle.quantize_cols(x)
+    _eq(s, sr, "row scales")
+    _eq(q, qr, "row codes")
+    _eq(st, str_, "col scales")
+    _eq(qt, qtr, "col codes")
+
+
+def test_swiglu_mx(oracle):
+    from kohakuwullm_amd.kernels.mxfp8.fused_act import swiglu_mx
+
+    g = _rand((200, 512), torch.bfloat16, 2.0, seed=3)
+    u = _rand((200, 512), torch.bfloat16, 1.0, seed=4)
+    q, s = swiglu_mx(g.to(DEV), u.to(DEV))
+    qr, sr = oracle.swiglu_quantize_rows(g, u)
+    q, s = q.view(torch.uint8).cpu(), s.cpu()
+    # the device sigmoid uses the hardware exp/rcp: an fp32 ulp can flip a rounding tie
+    assert (s != sr).float().mean() < 1e-3
+    assert (q != qr).float().mean() < 5e-3
+    act = g.float() * torch.sigmoid(g.float()) * u.float()
+    assert oracle.rel_error(oracle.dequant(q, s), act) < 0.04
+    # chunked halves of one projection, as GLUMLP produces them
+    both = torch.cat([g, u], dim=1).to(DEV)
+    gh, uh = both.chunk(2, dim=-1)
+    q2, s2 = swiglu_mx(gh, uh)
+    assert torch.equal(q2.view(torch.uint8).cpu(), q) and torch.equal(s2.cpu(), s)
+
+
+def test_full_size_properties(oracle):
+    """The 546M-dense activation shape: invariants that need no CPU pass over the whole tensor."""
+    mx = _mx()
+    g = torch.Generator().manual_seed(SEED)
+    x = torch.randn(16384, 1536, generator=g).bfloat16()
+    dev = x.to(DEV)
+    q, s, qt, st = mx.quantize_mx_dual(dev)
+    q1, s1 = mx.quantize_mx(dev)
+    qt1, st1 = mx.quantize_mx_cols(dev)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s, s1)
+    assert torch.equal(qt.view(torch.uint8), qt1.view(torch.uint8)) and torch.equal(st, st1)
+    # columns == rows of the materialised transpose
+    q2, s2 = mx.quantize_mx(dev.t().contiguous())
+    assert torch.equal(qt.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(st, s2)
+    # a seeded row sample against the oracle
+    rows = torch.randint(0, 16384, (64,), generator=g)
+    qr, sr = oracle.quantize_rows(x[rows].contiguous())
+    _eq(q[rows.to(DEV)], qr, "sampled codes")
+    _eq(s[rows.to(DEV)], sr, "sampled scales")
+    # block amax lands in the top binade of its scale
+    deq = q.float().reshape(16384, -1, 32).abs().amax(-1)
+    assert (deq <= 448).all() and (deq >= 224).all()
