@@ -89,6 +89,29 @@ int mx_swiglu_quantize_rows(const void *gate, const void *up, int dtype, int64_t
                             int64_t ldu, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream);
 
 /*
+ * h = silu(gate) * up taken from the fused input-projection output gu (M,2H), gate half
+ * first, row pitch ldgu; h is quantized along both axes in one pass: (q,s) (M,H) blocks
+ * along H for the output projection's forward, (qT,sT) (H,M) blocks along M for its wgrad.
+ * M % 32 == 0, H % 32 == 0.  The dense-MLP form of swiglu_mx (fused_act.py:69-101) for
+ * GLUMLP's fused w_in layout (src/kohakuwullm/models/components/mlp.py:61-73).
+ */
+int mx_swiglu_quantize_dual(const void *gu, int dtype, int64_t M, int64_t H, int64_t ldgu,
+                            uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
+                            uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
+
+/*
+ * SwiGLU backward fused with both quantizers: from dh (M,H) and the saved gu (M,2H),
+ * dgate = dh * up * sig * (1 + gate * (1 - sig)), dup = dh * gate * sig with sig =
+ * sigmoid(gate), all in fp32; dpre = [dgate | dup] (M,2H) is emitted only in MXFP8:
+ * (q,s) blocks along 2H for the input projection's dgrad and (qT,sT) (2H,M) blocks along
+ * M for its wgrad.  Closed form as src/kohakuwullm/kernels/elementwise/swiglu.py:108-119
+ * and experts_bwd.py:145-148.  M % 32 == 0, H % 32 == 0.
+ */
+int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, int64_t ldgu, int dtype,
+                                int64_t M, int64_t H, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
+                                uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
+
+/*
  * C (M,N) = deq(A) deq(B)^T, fp32 accumulate, cast to c_dtype (round to nearest
  * even).  A: codes (M,K) pitch lda + scales (M,K/32) pitch ldas; B: codes (N,K)
  * pitch ldb + scales (N,K/32) pitch ldbs; both K-minor.  K % 32 == 0.

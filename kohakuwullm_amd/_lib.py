@@ -31,6 +31,9 @@ SIGNATURES = {
     "mx_quantize_cols": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
     "mx_swiglu_quantize_rows": (_ci, [_p, _p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_swiglu_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_swiglu_bwd_quantize_dual": (
+        _ci, [_p, _i64, _p, _i64, _ci, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
     "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),
 }
 
@@ -79,3 +82,23 @@ def require_gpu(t: torch.Tensor, name: str) -> None:
         raise MXFP8LibraryError(
             f"{name} lives on {t.device}: the MXFP8 kernels run on an MI355X (gfx950) only and have no CPU path"
         )
+
+
+# Optional per-call device timing, used by the benchmark's roofline pass only.  When a list is
+# installed here every entry point call is bracketed by two events on the launch stream and
+# (name, work, start, end) is appended; `work` is the caller's algorithmic byte/flop count.
+TIMER: list | None = None
+
+
+def invoke(name: str, work: float, tensor: torch.Tensor, *args) -> None:
+    """Call entry point ``name`` with ``args`` on ``tensor``'s current stream and check its status."""
+    fn = getattr(load(), name)
+    if TIMER is None:
+        check(fn(*args, stream_of(tensor)), name)
+        return
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    status = fn(*args, stream_of(tensor))
+    end.record()
+    check(status, name)
+    TIMER.append((name, work, start, end))

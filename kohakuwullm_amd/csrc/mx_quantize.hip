@@ -121,38 +121,34 @@ __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__r
 #define QC_TILE 128
 #define QC_PITCH 136  // bytes per transposed LDS row (8-byte aligned, staggers banks)
 
-template <int DT, bool DUAL>
-__global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict__ x, int64_t M, int64_t K, int64_t ldx,
-                                                          uint8_t *__restrict__ qT, int64_t ldqT,
-                                                          uint8_t *__restrict__ sT, int64_t ldsT,
-                                                          uint8_t *__restrict__ q, int64_t ldq,
-                                                          uint8_t *__restrict__ s, int64_t lds, int pack_row_scales,
-                                                          int pack_col_scales) {
-    typedef typename Elem<DT>::type T;
-    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
-    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+struct QuantTileOut {
+    uint8_t *qT;  // (K,M) codes, blocks along M
+    int64_t ldqT;
+    uint8_t *sT;  // (K,M/32)
+    int64_t ldsT;
+    uint8_t *q;  // (M,K) codes, blocks along K (only when ROWS)
+    int64_t ldq;
+    uint8_t *s;  // (M,K/32)
+    int64_t lds;
+    int pack_row_scales, pack_col_scales;
+};
 
+// Quantizes the 128 x 128 tile held as v[8][8] per thread (rows m0 + rg*8 + i, columns
+// kc0 + cg*8 + c of the OUTPUT matrix, which has K columns and M rows) along the column
+// axis, and along the row axis too when ROWS.  `tile`/`tscale` are the workgroup's LDS
+// staging buffers; the caller must not touch them until the function's trailing barrier.
+template <bool ROWS>
+__device__ __forceinline__ void quant_tile(float (&v)[8][8], const QuantTileOut &o, int64_t M, int64_t K, int64_t m0,
+                                           int64_t kc0, uint8_t *tile, uint8_t *tscale) {
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
     const int cg = t & 15, rg = t >> 4;
-    const int64_t m0 = (int64_t)blockIdx.y * QC_TILE, k0 = (int64_t)blockIdx.x * QC_TILE;
-    const int64_t col = k0 + cg * 8;
+    const int64_t col = kc0 + cg * 8;
     const int64_t row0 = m0 + rg * 8;
-    const bool col_ok = col < K;                     // K % 8 == 0: an 8-column chunk is in or out
-    const bool blk_ok = m0 + wave * 32 < M;          // M % 32 == 0: a 32-row block is in or out
+    const bool col_ok = col < K;
+    const bool blk_ok = m0 + wave * 32 < M;
 
-    float v[8][8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        if (col_ok && blk_ok) {
-            Elem<DT>::load8((const T *)x + (row0 + i) * ldx + col, v[i]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
-        }
-    }
-
-    if (DUAL) {
+    if (ROWS) {
         // Row-axis outputs: the 4 lanes of a quad hold 32 consecutive columns of a row.
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -164,10 +160,10 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict_
                 v2i codes;
                 codes[0] = (int)pack4_e4m3(v[i][0] * inv, v[i][1] * inv, v[i][2] * inv, v[i][3] * inv);
                 codes[1] = (int)pack4_e4m3(v[i][4] * inv, v[i][5] * inv, v[i][6] * inv, v[i][7] * inv);
-                *(v2i *)(q + (row0 + i) * ldq + col) = codes;
-                uint8_t *sp = s + (row0 + i) * lds + (col >> 5);
-                bool full = k0 + QC_TILE <= K;
-                if (pack_row_scales && full) {
+                *(v2i *)(o.q + (row0 + i) * o.ldq + col) = codes;
+                uint8_t *sp = o.s + (row0 + i) * o.lds + (col >> 5);
+                bool full = kc0 + QC_TILE <= K;
+                if (o.pack_row_scales && full) {
                     if (cg == 0) *(uint32_t *)sp = packed;
                 } else if ((cg & 3) == 0) {
                     *sp = (uint8_t)byte;
@@ -205,26 +201,131 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict_
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         int kr = j * 32 + (t >> 3), ch = t & 7;
-        if (k0 + kr < K && m0 + ch * 16 < M) {
+        if (kc0 + kr < K && m0 + ch * 16 < M) {
             const v2i *src = (const v2i *)(tile + kr * QC_PITCH + ch * 16);
-            v4i o;
+            v4i w;
             v2i a = src[0], b = src[1];
-            o[0] = a[0];
-            o[1] = a[1];
-            o[2] = b[0];
-            o[3] = b[1];
-            *(v4i *)(qT + (k0 + kr) * ldqT + m0 + ch * 16) = o;
+            w[0] = a[0];
+            w[1] = a[1];
+            w[2] = b[0];
+            w[3] = b[1];
+            *(v4i *)(o.qT + (kc0 + kr) * o.ldqT + m0 + ch * 16) = w;
         }
     }
-    if (t < QC_TILE && k0 + t < K) {
-        uint8_t *sp = sT + (k0 + t) * ldsT + (m0 >> 5);
+    if (t < QC_TILE && kc0 + t < K) {
+        uint8_t *sp = o.sT + (kc0 + t) * o.ldsT + (m0 >> 5);
         int64_t nb = (M - m0) >> 5;
-        if (pack_col_scales && nb >= 4) {
+        if (o.pack_col_scales && nb >= 4) {
             *(uint32_t *)sp = *(const uint32_t *)(tscale + t * 4);
         } else {
             for (int b = 0; b < 4 && b < nb; b++) sp[b] = tscale[t * 4 + b];
         }
     }
+    __syncthreads();
+}
+
+template <int DT, bool DUAL>
+__global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict__ x, int64_t M, int64_t K, int64_t ldx,
+                                                          QuantTileOut o) {
+    typedef typename Elem<DT>::type T;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+    const int t = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.y * QC_TILE, k0 = (int64_t)blockIdx.x * QC_TILE;
+    const int64_t col = k0 + (t & 15) * 8;
+    const int64_t row0 = m0 + (t >> 4) * 8;
+    const bool ok = col < K && m0 + (t >> 6) * 32 < M;  // K % 8 == 0 and M % 32 == 0
+    float v[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (ok) {
+            Elem<DT>::load8((const T *)x + (row0 + i) * ldx + col, v[i]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
+        }
+    }
+    quant_tile<DUAL>(v, o, M, K, m0, k0, tile, tscale);
+}
+
+__device__ __forceinline__ float sigmoid_fast(float x) { return __fdividef(1.0f, 1.0f + __expf(-x)); }
+
+// h = silu(g) * u from the fused projection output gu (M, 2H) (gate half first), quantized
+// along both axes: (q,s) (M,H) for the down projection's forward, (qT,sT) (H,M) for its wgrad.
+template <int DT>
+__global__ __launch_bounds__(256) void swiglu_quant_dual_kernel(const void *__restrict__ gu, int64_t M, int64_t H,
+                                                                 int64_t ldgu, QuantTileOut o) {
+    typedef typename Elem<DT>::type T;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+    const int t = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.y * QC_TILE, k0 = (int64_t)blockIdx.x * QC_TILE;
+    const int64_t col = k0 + (t & 15) * 8;
+    const int64_t row0 = m0 + (t >> 4) * 8;
+    const bool ok = col < H && m0 + (t >> 6) * 32 < M;
+    float v[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (ok) {
+            float g[8], u[8];
+            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + col, g);
+            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + H + col, u);
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = g[c] * sigmoid_fast(g[c]) * u[c];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
+        }
+    }
+    quant_tile<true>(v, o, M, H, m0, k0, tile, tscale);
+}
+
+// SwiGLU backward fused with both quantizers.  Reads dh (M,H) and the saved projection
+// output gu (M,2H); forms dgate = dh * u * s * (1 + g (1 - s)) and dup = dh * g * s with
+// s = sigmoid(g) in fp32 (elementwise/swiglu.py:108-119, experts_bwd.py:145-148 of the
+// reference); writes dpre = [dgate | dup] quantized along 2H ((q,s): (M,2H)) for the input
+// projection's dgrad and along M ((qT,sT): (2H,M)) for its wgrad.  o.q/o.qT address the
+// full (M,2H) / (2H,M) outputs.
+template <int DT>
+__global__ __launch_bounds__(256) void swiglu_bwd_quant_dual_kernel(const void *__restrict__ dh, int64_t lddh,
+                                                                     const void *__restrict__ gu, int64_t ldgu,
+                                                                     int64_t M, int64_t H, QuantTileOut o) {
+    typedef typename Elem<DT>::type T;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+    const int t = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.y * QC_TILE, k0 = (int64_t)blockIdx.x * QC_TILE;
+    const int64_t col = k0 + (t & 15) * 8;
+    const int64_t row0 = m0 + (t >> 4) * 8;
+    const bool ok = col < H && m0 + (t >> 6) * 32 < M;
+    float v[8][8], w[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (ok) {
+            float g[8], u[8], d[8];
+            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + col, g);
+            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + H + col, u);
+            Elem<DT>::load8((const T *)dh + (row0 + i) * lddh + col, d);
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                float sg = sigmoid_fast(g[c]);
+                v[i][c] = d[c] * u[c] * sg * (1.0f + g[c] * (1.0f - sg));
+                w[i][c] = d[c] * g[c] * sg;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = w[i][c] = 0.0f;
+        }
+    }
+    // The gate half occupies output columns [0,H), the up half [H,2H): same tile, shifted.
+    // Columns at or beyond H inside the gate-half tile are masked by passing K = H.
+    quant_tile<true>(v, o, M, H, m0, k0, tile, tscale);
+    QuantTileOut o2 = o;
+    o2.q += H;
+    o2.s += H / MX_BLOCK;
+    o2.qT += H * o.ldqT;
+    o2.sT += H * o.ldsT;
+    quant_tile<true>(w, o2, M, H, m0, k0, tile, tscale);
 }
 
 // ------------------------------------------------------------------------------------
@@ -332,15 +433,21 @@ static int launch_rows(const void *x, int64_t M, int64_t K, int64_t sx_row, int6
     return MX_OK;
 }
 
+static QuantTileOut tile_out(uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s,
+                             int64_t lds) {
+    QuantTileOut o;
+    o.qT = qT, o.ldqT = ldqT, o.sT = sT, o.ldsT = ldsT, o.q = q, o.ldq = ldq, o.s = s, o.lds = lds;
+    o.pack_row_scales = s != nullptr && aligned(s, 4) && lds % 4 == 0;
+    o.pack_col_scales = aligned(sT, 4) && ldsT % 4 == 0;
+    return o;
+}
+
 template <int DT, bool DUAL>
 static int launch_cols(const void *x, int64_t M, int64_t K, int64_t ldx, uint8_t *qT, int64_t ldqT, uint8_t *sT,
                        int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, hipStream_t st) {
     dim3 grid((unsigned)((K + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
     if (grid.y > 65535u) return MX_EUNSUPPORTED;
-    int pack_row = DUAL && aligned(s, 4) && lds % 4 == 0;
-    int pack_col = aligned(sT, 4) && ldsT % 4 == 0;
-    quant_cols_kernel<DT, DUAL><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, pack_row,
-                                                             pack_col);
+    quant_cols_kernel<DT, DUAL><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds));
     MX_LAUNCH_CHECK();
     return MX_OK;
 }
@@ -433,4 +540,46 @@ extern "C" int mx_swiglu_quantize_rows(const void *gate, const void *up, int dty
     hipStream_t st = (hipStream_t)stream;
     return dtype == MX_BF16 ? launch_swiglu<MX_BF16>(gate, up, M, K, ldg, ldu, q, ldq, s, lds, st)
                             : launch_swiglu<MX_FP16>(gate, up, M, K, ldg, ldu, q, ldq, s, lds, st);
+}
+
+extern "C" int mx_swiglu_quantize_dual(const void *gu, int dtype, int64_t M, int64_t H, int64_t ldgu, uint8_t *q,
+                                       int64_t ldq, uint8_t *s, int64_t lds, uint8_t *qT, int64_t ldqT, uint8_t *sT,
+                                       int64_t ldsT, void *stream) {
+    if (M < 0 || H < 0 || M % MX_BLOCK || H % MX_BLOCK || ldgu < 2 * H || ldq < H || lds < H / MX_BLOCK || ldqT < M ||
+        ldsT < M / MX_BLOCK)
+        return MX_EINVAL;
+    if (M == 0 || H == 0) return MX_OK;
+    if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
+    if (!aligned(gu, 16) || (ldgu * 2) % 16 || !aligned(q, 8) || ldq % 8 || !aligned(qT, 16) || ldqT % 16)
+        return MX_EUNSUPPORTED;
+    dim3 grid((unsigned)((H + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
+    if (grid.y > 65535u) return MX_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds);
+    if (dtype == MX_BF16) swiglu_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(gu, M, H, ldgu, o);
+    else swiglu_quant_dual_kernel<MX_FP16><<<grid, dim3(256), 0, st>>>(gu, M, H, ldgu, o);
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+extern "C" int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, int64_t ldgu, int dtype,
+                                           int64_t M, int64_t H, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
+                                           uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream) {
+    if (M < 0 || H < 0 || M % MX_BLOCK || H % MX_BLOCK || lddh < H || ldgu < 2 * H || ldq < 2 * H ||
+        lds < 2 * H / MX_BLOCK || ldqT < M || ldsT < M / MX_BLOCK)
+        return MX_EINVAL;
+    if (M == 0 || H == 0) return MX_OK;
+    if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
+    if (!aligned(gu, 16) || (ldgu * 2) % 16 || !aligned(dh, 16) || (lddh * 2) % 16 || !aligned(q, 8) || ldq % 8 ||
+        !aligned(qT, 16) || ldqT % 16)
+        return MX_EUNSUPPORTED;
+    dim3 grid((unsigned)((H + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
+    if (grid.y > 65535u) return MX_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds);
+    if (H % 128) o.pack_row_scales = 0;  // the up half's scale columns start at H/32: keep dword stores aligned
+    if (dtype == MX_BF16) swiglu_bwd_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);
+    else swiglu_bwd_quant_dual_kernel<MX_FP16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);
+    MX_LAUNCH_CHECK();
+    return MX_OK;
 }

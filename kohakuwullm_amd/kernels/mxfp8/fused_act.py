@@ -34,9 +34,9 @@ def swiglu_mx(gate: torch.Tensor, up: torch.Tensor):
     q = torch.empty(m, k, device=gate.device, dtype=torch.float8_e4m3fn)
     s = torch.empty(m, k // BLOCK_SCALE, device=gate.device, dtype=torch.uint8)
     if m and k:
-        rc = _lib.load().mx_swiglu_quantize_rows(
+        _lib.invoke(
+            "mx_swiglu_quantize_rows", m * k * (2 * gate.element_size() + 1 + 1 / BLOCK_SCALE), gate,
             g2.data_ptr(), u2.data_ptr(), _lib.MX_DTYPE[gate.dtype], m, k, g2.stride(0), u2.stride(0),
-            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE, _lib.stream_of(gate),
+            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE,
         )
-        _lib.check(rc, "mx_swiglu_quantize_rows")
     return q, s

@@ -1,0 +1,152 @@
+"""MXFP8 linear: fp8 FPROP, DGRAD and WGRAD on the gfx950 block-scaled MFMA GEMM.
+
+Same surface as the reference's ``MXFP8Linear``
+(``src/kohakuwullm/kernels/mxfp8/linear.py:77-126``): a bias-free ``nn.Linear`` stand-in
+whose quantized weight copies are plain attributes (never buffers, so they stay out of
+``state_dict``), rebuilt by ``refresh_quantized_weight()`` after every optimizer step and
+dropped by any ``_apply``.  ``in_features`` must be a multiple of 128; ``out_features`` is
+zero-padded to one for DGRAD's contraction, which is exact.  Compute and output dtype
+follow autocast, never the weight.
+
+One difference from the reference, on purpose: WGRAD also runs in MXFP8
+(``dW = Qcol(dY) . Qcol(X)^T`` with 32-token blocks), where the reference multiplies in
+16 bits (``linear.py:72-73``).  It falls back to that 16-bit product only when the token
+count is not a multiple of 32.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from kohakuwullm_amd.kernels.mxfp8.quantize import (
+    BLOCK_SCALE,
+    mxfp8_matmul_pq,
+    quantize_mx,
+    quantize_mx_cols,
+    quantize_mx_dual,
+)
+
+# Alignment of FPROP's contraction axis (kept at the reference's value so `swap_mxfp8`
+# accepts and refuses exactly the same layers).
+VENDOR_K_ALIGN = 128
+
+
+def compute_dtype(x: torch.Tensor) -> torch.dtype:
+    """The dtype ``nn.Linear`` would compute in for this input (autocast, else the input's)."""
+    if torch.is_autocast_enabled("cuda"):
+        return torch.get_autocast_dtype("cuda")
+    return x.dtype
+
+
+class _PadLastAxis:
+    """Zero-pads the last axis by ``width`` columns; ``width == 0`` returns the tensor itself.
+
+    A picklable callable: the module that owns it must survive ``copy.deepcopy`` and
+    ``torch.save``.
+    """
+
+    __slots__ = ("width",)
+
+    def __init__(self, width: int) -> None:
+        self.width = int(width)
+
+    def __call__(self, tensor: torch.Tensor) -> torch.Tensor:
+        return F.pad(tensor, (0, self.width)) if self.width else tensor
+
+
+class _MXFP8Linear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, wq_f, ws_f, wq_d, ws_d, pad_k):
+        compute = compute_dtype(x)
+        shape = x.shape
+        x2d = x.reshape(-1, shape[-1]).to(compute)
+        if x2d.stride(-1) != 1:
+            x2d = x2d.contiguous()
+        need_dw = ctx.needs_input_grad[1]
+        fp8_wgrad = need_dw and x2d.shape[0] % BLOCK_SCALE == 0 and x2d.shape[0] > 0
+        if fp8_wgrad:
+            # One pass over x gives FPROP's operand and WGRAD's (blocks along tokens).
+            xq, xs, xtq, xts = quantize_mx_dual(x2d)
+            saved_x = (xtq, xts)
+        else:
+            xq, xs = quantize_mx(x2d)
+            saved_x = (x2d if need_dw else None, None)
+        out = mxfp8_matmul_pq(xq, xs, wq_f, ws_f, compute)
+        ctx.save_for_backward(*saved_x, wq_d, ws_d)
+        ctx.fp8_wgrad = fp8_wgrad
+        ctx.pad_k = pad_k
+        ctx.x_dtype = x.dtype
+        ctx.compute = compute
+        ctx.out_features = weight.shape[0]
+        return out.reshape(*shape[:-1], out.shape[-1])
+
+    @staticmethod
+    def backward(ctx, dout):
+        x_a, x_b, wq_d, ws_d = ctx.saved_tensors
+        shape = dout.shape
+        d2d = dout.reshape(-1, shape[-1]).to(ctx.compute).contiguous()
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        dx = dw = None
+        padded = ctx.pad_k(d2d)
+        if need_dw and ctx.fp8_wgrad:
+            dq, ds, dtq, dts = quantize_mx_dual(padded)
+            n = ctx.out_features
+            # dW (out,in) = dY^T (out,tokens) . (X^T (in,tokens))^T, contraction over tokens.
+            dw = mxfp8_matmul_pq(dtq[:n], dts[:n], x_a, x_b, ctx.compute)
+        else:
+            dq, ds = quantize_mx(padded) if need_dx else (None, None)
+            if need_dw:
+                dw = d2d.t() @ x_a
+        if need_dx:
+            dx = mxfp8_matmul_pq(dq, ds, wq_d, ws_d, ctx.x_dtype)
+            dx = dx.reshape(*shape[:-1], dx.shape[-1])
+        return dx, dw, None, None, None, None, None
+
+
+class MXFP8Linear(torch.nn.Module):
+    """``nn.Linear`` (no bias) computing FPROP, DGRAD and WGRAD in MXFP8.
+
+    ``refresh_quantized_weight`` must be called after every optimizer step.  ``dw`` comes
+    back in the compute dtype and autograd casts it during accumulation.
+    """
+
+    def __init__(self, in_features: int, out_features: int, dtype=torch.bfloat16):
+        super().__init__()
+        if in_features % VENDOR_K_ALIGN:
+            raise ValueError(
+                f"in_features={in_features} must be a multiple of {VENDOR_K_ALIGN}; "
+                "it is FPROP's contraction axis and is shared with the activation "
+                "cast, so it cannot be padded without padding every input"
+            )
+        self.in_features = in_features
+        self.out_features = out_features
+        padded = -(-out_features // VENDOR_K_ALIGN) * VENDOR_K_ALIGN
+        self.padded_out_features = padded
+        self._pad_k = _PadLastAxis(padded - out_features)
+        self.weight = torch.nn.Parameter(torch.empty(out_features, in_features, dtype=dtype))
+        torch.nn.init.normal_(self.weight, std=in_features**-0.5)
+        self._cache: tuple[torch.Tensor, ...] | None = None
+
+    @torch.no_grad()
+    def refresh_quantized_weight(self) -> None:
+        wq_f, ws_f = quantize_mx(self.weight)
+        if self._pad_k.width == 0:
+            # Blocks along out_features without materialising the transpose.
+            wq_d, ws_d = quantize_mx_cols(self.weight)
+        else:
+            wq_d, ws_d = quantize_mx(self._pad_k(self.weight.t()))
+        self._cache = (wq_f, ws_f, wq_d, ws_d)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self._cache is None:
+            self.refresh_quantized_weight()
+        return _MXFP8Linear.apply(x, self.weight, *self._cache, self._pad_k)
+
+    def _apply(self, *args, **kwargs):
+        """Any device or dtype transform drops the quantized cache; ``forward`` rebuilds it."""
+        self._cache = None
+        return super()._apply(*args, **kwargs)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, mxfp8=True"

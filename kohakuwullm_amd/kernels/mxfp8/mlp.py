@@ -1,0 +1,114 @@
+"""Dense SwiGLU feed-forward in MXFP8 with the activation fused into the quantizers.
+
+The reference's dense ``GLUMLP`` runs ``w_out(silu(gate) * value)`` as two ``MXFP8Linear``
+calls around an eager 16-bit activation (``src/kohakuwullm/models/components/mlp.py:68-73``)
+and names the fused cast ``swiglu_mx`` (``kernels/mxfp8/fused_act.py:69-101``) as the
+producer epilogue it wants.  This function is that fusion for the whole layer:
+
+forward   X --dual quantize--> GU = Xq . Wq_in^T --SwiGLU + dual quantize--> Y = Hq . Wq_out^T
+backward  dY --dual quantize--> dH = dYq . Wq_out_d^T --SwiGLU' + dual quantize--> dX = dPq . Wq_in_d^T
+          dW_out = dY^T . H^T-blocks,  dW_in = dP^T . X^T-blocks   (contraction over tokens)
+
+``h`` and ``dpre`` never exist in 16 bits: the SwiGLU kernels read the GEMM output once and
+emit the row-blocked operand for the next GEMM and the token-blocked operand for WGRAD.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kohakuwullm_amd import _lib
+from kohakuwullm_amd.kernels.mxfp8.linear import compute_dtype
+from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE, mxfp8_matmul_pq, quantize_mx_dual
+
+_FP8 = torch.float8_e4m3fn
+
+
+def swiglu_mx_dual(gu: torch.Tensor):
+    """``h = silu(gu[:, :H]) * gu[:, H:]`` as ``(q, s, qT, sT)``: blocks along H and along tokens."""
+    m, two_h = gu.shape
+    h = two_h // 2
+    if two_h % 2 or h % BLOCK_SCALE or m % BLOCK_SCALE:
+        raise ValueError(f"gu {tuple(gu.shape)}: tokens and hidden must be multiples of {BLOCK_SCALE}")
+    _lib.require_gpu(gu, "gu")
+    q = torch.empty(m, h, device=gu.device, dtype=_FP8)
+    s = torch.empty(m, h // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
+    qt = torch.empty(h, m, device=gu.device, dtype=_FP8)
+    st = torch.empty(h, m // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
+    _lib.invoke(
+        "mx_swiglu_quantize_dual", m * h * (2 * gu.element_size() + 2 * (1 + 1 / BLOCK_SCALE)), gu,
+        gu.data_ptr(), _lib.MX_DTYPE[gu.dtype], m, h, gu.stride(0), q.data_ptr(), h, s.data_ptr(), h // BLOCK_SCALE,
+        qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE,
+    )
+    return q, s, qt, st
+
+
+def swiglu_bwd_mx_dual(dh: torch.Tensor, gu: torch.Tensor):
+    """SwiGLU backward emitted straight in MXFP8: ``dpre = [dgate | dup]`` as ``(q, s, qT, sT)``."""
+    m, two_h = gu.shape
+    h = two_h // 2
+    if dh.shape != (m, h) or h % BLOCK_SCALE or m % BLOCK_SCALE:
+        raise ValueError(f"dh {tuple(dh.shape)} does not match gu {tuple(gu.shape)}")
+    _lib.require_gpu(gu, "gu")
+    q = torch.empty(m, two_h, device=gu.device, dtype=_FP8)
+    s = torch.empty(m, two_h // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
+    qt = torch.empty(two_h, m, device=gu.device, dtype=_FP8)
+    st = torch.empty(two_h, m // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
+    _lib.invoke(
+        "mx_swiglu_bwd_quantize_dual", m * h * (3 * gu.element_size() + 4 * (1 + 1 / BLOCK_SCALE)), gu,
+        dh.data_ptr(), dh.stride(0), gu.data_ptr(), gu.stride(0), _lib.MX_DTYPE[gu.dtype], m, h,
+        q.data_ptr(), two_h, s.data_ptr(), two_h // BLOCK_SCALE, qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE,
+    )
+    return q, s, qt, st
+
+
+class _MXFP8SwiGLUMLP(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w_in, w_out, in_f, in_d, out_f, out_d):
+        compute = compute_dtype(x)
+        shape = x.shape
+        x2d = x.reshape(-1, shape[-1]).to(compute)
+        if x2d.stride(-1) != 1:
+            x2d = x2d.contiguous()
+        xq, xs, xtq, xts = quantize_mx_dual(x2d)
+        gu = mxfp8_matmul_pq(xq, xs, *in_f, compute)
+        hq, hs, htq, hts = swiglu_mx_dual(gu)
+        y = mxfp8_matmul_pq(hq, hs, *out_f, compute)
+        if any(ctx.needs_input_grad):
+            ctx.save_for_backward(xtq, xts, gu, htq, hts, *in_d, *out_d)
+            ctx.compute = compute
+            ctx.x_dtype = x.dtype
+        return y.reshape(*shape[:-1], y.shape[-1])
+
+    @staticmethod
+    def backward(ctx, dout):
+        xtq, xts, gu, htq, hts, win_dq, win_ds, wout_dq, wout_ds = ctx.saved_tensors
+        shape = dout.shape
+        d2d = dout.reshape(-1, shape[-1]).to(ctx.compute).contiguous()
+        dq, ds, dtq, dts = quantize_mx_dual(d2d)
+        dh = mxfp8_matmul_pq(dq, ds, wout_dq, wout_ds, ctx.compute)
+        pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu)
+        dx = dw_in = dw_out = None
+        if ctx.needs_input_grad[0]:
+            dx = mxfp8_matmul_pq(pq, ps, win_dq, win_ds, ctx.x_dtype).reshape(*shape[:-1], -1)
+        if ctx.needs_input_grad[1]:
+            dw_in = mxfp8_matmul_pq(ptq, pts, xtq, xts, ctx.compute)
+        if ctx.needs_input_grad[2]:
+            dw_out = mxfp8_matmul_pq(dtq, dts, htq, hts, ctx.compute)
+        return dx, dw_in, dw_out, None, None, None, None
+
+
+def mxfp8_swiglu_mlp(x, w_in, w_out, packed) -> torch.Tensor:
+    """``(silu(x W_g^T) * (x W_u^T)) W_out^T`` with ``w_in = [W_g; W_u]`` ``(2H, dim)``, ``w_out`` ``(dim, H)``.
+
+    ``packed`` is ``(in_fwd, in_dgrad, out_fwd, out_dgrad)``, each a ``(codes, scales)`` pair:
+    the weights blocked along their contraction axis for FPROP and along the other axis for
+    DGRAD.  ``w_in``/``w_out`` are passed so autograd routes ``dW`` to the master parameters.
+    Tokens, ``dim`` and ``H`` must be multiples of 32.
+    """
+    tokens = x.numel() // x.shape[-1]
+    if tokens % BLOCK_SCALE:
+        raise ValueError(f"token count {tokens} must be a multiple of {BLOCK_SCALE} for the MXFP8 WGRAD")
+    if w_in.shape[0] != 2 * w_out.shape[1] or w_in.shape[1] != x.shape[-1] or w_out.shape[0] != x.shape[-1]:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w_in {tuple(w_in.shape)}, w_out {tuple(w_out.shape)}")
+    return _MXFP8SwiGLUMLP.apply(x, w_in, w_out, *packed)

@@ -44,11 +44,11 @@ def quantize_mx(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     q = torch.empty(m, k, device=x.device, dtype=_FP8)
     s = torch.empty(m, k // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
     if m and k:
-        rc = _lib.load().mx_quantize_rows(
+        _lib.invoke(
+            "mx_quantize_rows", m * k * (x.element_size() + 1 + 1 / BLOCK_SCALE), x,
             x.data_ptr(), _lib.MX_DTYPE[x.dtype], m, k, x.stride(0), x.stride(1),
-            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE, _lib.stream_of(x),
+            q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE,
         )
-        _lib.check(rc, "mx_quantize_rows")
     return q, s
 
 
@@ -67,11 +67,11 @@ def quantize_mx_cols(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     qt = torch.empty(k, m, device=x.device, dtype=_FP8)
     st = torch.empty(k, m // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
     if m and k:
-        rc = _lib.load().mx_quantize_cols(
+        _lib.invoke(
+            "mx_quantize_cols", m * k * (x.element_size() + 1 + 1 / BLOCK_SCALE), x,
             x.data_ptr(), _lib.MX_DTYPE[x.dtype], m, k, x.stride(0),
-            qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE, _lib.stream_of(x),
+            qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE,
         )
-        _lib.check(rc, "mx_quantize_cols")
     return qt, st
 
 
@@ -92,24 +92,24 @@ def quantize_mx_dual(x: torch.Tensor):
     qt = torch.empty(k, m, device=x.device, dtype=_FP8)
     st = torch.empty(k, m // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
     if m and k:
-        rc = _lib.load().mx_quantize_dual(
+        _lib.invoke(
+            "mx_quantize_dual", m * k * (x.element_size() + 2 * (1 + 1 / BLOCK_SCALE)), x,
             x.data_ptr(), _lib.MX_DTYPE[x.dtype], m, k, x.stride(0),
             q.data_ptr(), k, s.data_ptr(), k // BLOCK_SCALE,
-            qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE, _lib.stream_of(x),
+            qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE,
         )
-        _lib.check(rc, "mx_quantize_dual")
     return q, s, qt, st
 
 
 def _gemm_nt_into(aq, a_scale, bq, b_scale, out) -> None:
     m, k = aq.shape
     n = bq.shape[0]
-    rc = _lib.load().mx_gemm_nt(
+    _lib.invoke(
+        "mx_gemm_nt", 2.0 * m * n * k, aq,
         aq.data_ptr(), a_scale.data_ptr(), bq.data_ptr(), b_scale.data_ptr(), out.data_ptr(),
         _lib.MX_DTYPE[out.dtype], m, n, k, aq.stride(0), a_scale.stride(0), bq.stride(0), b_scale.stride(0),
-        out.stride(0), 0, _lib.stream_of(aq),
+        out.stride(0), 0,
     )
-    _lib.check(rc, "mx_gemm_nt")
 
 
 def mxfp8_matmul_pq(
