@@ -38,8 +38,12 @@ enum mx_dtype { MX_BF16 = 0, MX_FP16 = 1, MX_FP32 = 2 };
 
 /* Epilogues of the GEMM entry points. */
 enum mx_epilogue {
-    MX_EPI_NONE = 0 /* C = A B^T, cast to c_dtype */
+    MX_EPI_NONE = 0,      /* C = A B^T, cast to c_dtype */
+    MX_EPI_ACCUMULATE = 1 /* C += A B^T with fp32 atomic adds; c_dtype must be MX_FP32 */
 };
+/* OR into `epilogue` to cut K into n slices that run as independent tiles (needs
+ * MX_EPI_ACCUMULATE and a caller-zeroed C): fills the GPU when M*N alone gives too few tiles. */
+#define MX_EPI_SPLIT_K(n) ((n) << 8)
 
 int mx_abi_version(void);
 const char *mx_strerror(int status);

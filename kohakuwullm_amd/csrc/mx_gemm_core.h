@@ -1,0 +1,504 @@
+// Core of the MXFP8 NT GEMM kernels for gfx950: tile shape, LDS layout, the K-stage body on
+// v_mfma_scale_f32_16x16x128_f8f6f4 and the persistent tile loop.  Dense, grouped and
+// expert kernels plug a "problem" policy (tile iterator, operand addressing, epilogue)
+// into persistent_gemm().
+//
+// Shape of the kernel
+//   * workgroup tile BM x BN x 128, 64-lane waves arranged WGM x WGN, each wave owning a
+//     (BM/WGM) x (BN/WGN) sub-tile as 16x16 MFMA accumulators;
+//   * one workgroup per CU, persistent: it walks a strided list of tiles and issues the
+//     first operand stage (and scales) of the next tile before the epilogue of the current
+//     one, so HBM latency, the epilogue and workgroup dispatch never sit between two tiles;
+//   * operand tiles travel HBM -> LDS with the direct global-to-LDS load (16 bytes per lane,
+//     each lane supplying its own global address, which is what makes row gathers free),
+//     double buffered, one workgroup barrier per 128-wide K stage;
+//   * operand layout of the scaled 16x16x128 MFMA (measured on gfx950): lane (r = l%16,
+//     g = l/16) holds row r; its first 16 bytes belong to MX block g>>1 and its last 16 bytes
+//     to MX block 2 + (g>>1) of the 128-wide K step, and the scale of (row r, block b) is read
+//     from lane r + 16 b.  So a lane loads K bytes [16g,16g+16) and [64+16g,64+16g+16) and
+//     supplies the scale byte of block g;
+//   * LDS rows are 128 bytes with the 16-byte chunks XOR-swizzled so that the 16 lanes of
+//     an MFMA row group read 16 different bank quads;
+//   * scales are fetched once per 512 of K (16 bytes per row), byte-transposed 4x4 and
+//     parked in LDS so a lane reads ONE dword per sub-tile per 4 stages and the stage picks
+//     its byte with the instruction's op_sel: no VALU work on scales in the main loop;
+//   * the MFMA is issued "B rows x A rows", so a lane's 4 accumulator registers are 4
+//     consecutive N of one output row; the B rows feeding sub-tiles 4j..4j+3 are permuted so
+//     that sub-tiles (4j, 4j+1) give a lane 8 consecutive N and the four lanes sharing an
+//     output row cover 32 consecutive N between them (sub-tiles (4j+2, 4j+3): the next 32).
+//     One 16-byte store per lane then writes 64 contiguous bytes per output row; a layout
+//     that leaves gaps between the lanes' pieces is issue-bound at ~16 B/clk.
+#pragma once
+
+#include "mx_common.h"
+
+#ifndef MX_L2_AHEAD
+#define MX_L2_AHEAD 0
+#endif
+
+namespace mx {
+
+typedef __attribute__((address_space(1))) const void gptr_t;
+typedef __attribute__((address_space(3))) void lptr_t;
+
+// Direct global-to-LDS copy of 16 bytes per lane.  `base` (wave-uniform, in scalar registers)
+// plus the lane's 32-bit byte offset is the global address; the wave's 64 x 16 bytes land
+// contiguously in LDS at byte address `lds` (wave-uniform, goes through M0).
+// Written as inline asm on purpose: the kernel orders these copies against LDS reads itself,
+// with explicit vmcnt waits and workgroup barriers, and lets chosen younger operations (L2
+// touches, epilogue stores) stay in flight across a barrier; the compiler's own accounting
+// would insert a full vmcnt(0) before every LDS read that follows a copy it can see.
+__device__ __forceinline__ void dma16(const uint8_t *base, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(lds)
+                 : "memory");
+}
+
+// One 4-byte direct-to-LDS load per lane whose only purpose is to pull the 128-byte line at
+// `g` into L2 ahead of the stage that needs it; the 256 bytes it deposits in LDS are junk.
+__device__ __forceinline__ void l2_touch(const uint8_t *g, uint32_t lds_junk) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(lds_junk) : "memory");
+}
+
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    uint64_t u = (uint64_t)p;
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
+    uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+}
+
+template <int BM_, int BN_, int WGM_, int WGN_>
+struct GemmShape {
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
+    static constexpr int BK = 128;
+    static constexpr int NW = WGM * WGN;
+    static constexpr int NTHR = NW * 64;
+    static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    static constexpr int MT = WTM / 16, NT = WTN / 16;
+    static constexpr int QA = BM / 8 / NW, QB = BN / 8 / NW;  // DMA instructions per wave per stage
+    static constexpr int DATA_A = BM * BK, DATA_B = BN * BK;  // bytes per stage
+    // Scale planes [buffer][g][row] of dwords; the plane pitch is padded so the 64 lanes of
+    // a wave (16 rows x 4 planes) read 64 different banks.
+    static constexpr int PA = BM + 16, PB = BN + 32;
+    static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
+    static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B) + NW * 256;
+    static constexpr bool TWO_ROWS = BM + BN > NTHR;
+    static_assert(WTN % 64 == 0, "a wave's N extent must be a multiple of 64");
+    static_assert(WTM % 16 == 0, "a wave's M extent must be a multiple of 16");
+    static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "DMA rows must divide over the waves");
+    static_assert(BM + BN <= 2 * NTHR, "scale loader assumes at most two rows per thread");
+};
+
+// chunk swizzles: position of logical 16-byte chunk c of LDS row r is c ^ swz(r)
+__device__ __forceinline__ int swz_a(int r) { return (r >> 1) & 7; }
+__device__ __forceinline__ int swz_b(int r) { return (((r >> 3) & 3) << 1) | ((r >> 1) & 1); }
+
+// 4x4 byte transpose: in d[s] = bytes {4s+0..4s+3}; out t[g] = bytes {g, 4+g, 8+g, 12+g}.
+__device__ __forceinline__ void transpose4x4(const uint32_t (&d)[4], uint32_t (&t)[4]) {
+    // v_perm_b32(a, b, sel): byte i of the result is byte sel[i] of the 8-byte {a:b} (b = bytes 0-3).
+    uint32_t p01l = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u);  // d0.b0 d1.b0 d0.b1 d1.b1
+    uint32_t p01h = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);  // d0.b2 d1.b2 d0.b3 d1.b3
+    uint32_t p23l = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+    uint32_t p23h = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+    t[0] = __builtin_amdgcn_perm(p23l, p01l, 0x05040100u);  // lo16(p01l) lo16(p23l)
+    t[1] = __builtin_amdgcn_perm(p23l, p01l, 0x07060302u);  // hi16(p01l) hi16(p23l)
+    t[2] = __builtin_amdgcn_perm(p23h, p01h, 0x05040100u);
+    t[3] = __builtin_amdgcn_perm(p23h, p01h, 0x07060302u);
+}
+
+// Where the lane sits: which wave, and its (row-in-16, K-group) role in the MFMA operands.
+struct Lane {
+    int tid, lane, wave, wm, wn, r16, g;
+};
+
+template <typename S>
+__device__ __forceinline__ Lane lane_of() {
+    Lane L;
+    L.tid = threadIdx.x;
+    L.lane = L.tid & 63;
+    L.wave = __builtin_amdgcn_readfirstlane(L.tid >> 6);
+    L.wm = L.wave / S::WGN;
+    L.wn = L.wave % S::WGN;
+    L.r16 = L.lane & 15;
+    L.g = L.lane >> 4;
+    return L;
+}
+
+// Offset, inside a wave's 64-row slice of the B tile, of the rows feeding sub-tile j.
+__device__ __forceinline__ constexpr int b_sub_off(int j) { return (j >> 2) * 64 + ((j & 3) >> 1) * 32 + (j & 1) * 4; }
+
+// Row of the B tile (0..BN-1) that feeds accumulator sub-tile j, MFMA row rr (0..15), for a
+// wave at column wn.  Output column of accumulator register v of lane group g, sub-tile j:
+// wn*WTN + b_sub_off(j) + 8 g + v.
+template <typename S>
+__device__ __forceinline__ int b_tile_row(int wn, int j, int rr) {
+    return wn * S::WTN + b_sub_off(j) + 8 * (rr >> 2) + (rr & 3);
+}
+
+// Everything the copy engine needs for one tile: where A and B rows come from and where
+// this thread's scale rows live.  `a_voff`/`b_voff` are byte offsets of this lane's 16-byte
+// chunk of each DMA instruction relative to the (wave-uniform) bases, for K = 0.
+template <typename S>
+struct IssueCtx {
+    const uint8_t *a_base, *b_base;
+    uint32_t a_voff[S::QA], b_voff[S::QB];
+    const uint8_t *srow0, *srow1;  // scale rows tid and tid + NTHR of the [A rows; B rows] list
+    int kt0, kt1;                  // K range in 128-byte stages (absolute)
+};
+
+// Row r (0..BM-1) of the A tile and row r of the B tile as the DMA engine sees them.
+template <typename S>
+__device__ __forceinline__ int dma_row(const Lane &L, int q) { return (q * S::NW + L.wave) * 8 + (L.lane >> 3); }
+
+// A copy of the lane descriptor the optimiser cannot see through: address arithmetic done on
+// it inside the per-tile setup is recomputed once per tile instead of being hoisted out of
+// the tile loop and kept in (spilled) registers across the K loop.
+__device__ __forceinline__ Lane opaque(const Lane &L) {
+    Lane R = L;
+    asm volatile("" : "+v"(R.tid), "+v"(R.lane));
+    return R;
+}
+
+template <typename S>
+__device__ __forceinline__ void issue_stage(const IssueCtx<S> &c, const Lane &L, int kt, uint8_t *ldsA, uint8_t *ldsB,
+                                            int buf) {
+    // The stage's base address is forced into SGPRs so each load is "scalar base + 32-bit
+    // lane offset" and costs no 64-bit vector address arithmetic.
+    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt * 128);
+    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt * 128);
+    const uint32_t la = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf * S::DATA_A + L.wave * 1024);
+    const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf * S::DATA_B + L.wave * 1024);
+#pragma unroll
+    for (int q = 0; q < S::QA; q++) dma16(ga, c.a_voff[q], la + q * S::NW * 1024);
+#pragma unroll
+    for (int q = 0; q < S::QB; q++) dma16(gb, c.b_voff[q], lb + q * S::NW * 1024);
+}
+
+// 16 scale bytes (4 stages x 4 blocks) of one row starting at scale column kb0.
+template <bool K512>
+__device__ __forceinline__ void load_scales(const uint8_t *row, int kb0, int kb_end, uint32_t (&d)[4]) {
+    const uint8_t *p = row + kb0;
+    if (K512) {
+        v4i t = *(const v4i *)p;
+        d[0] = t[0], d[1] = t[1], d[2] = t[2], d[3] = t[3];
+    } else {
+#pragma unroll
+        for (int s = 0; s < 4; s++) d[s] = kb0 + 4 * s < kb_end ? *(const uint32_t *)(p + 4 * s) : 0u;
+    }
+}
+
+template <typename S>
+__device__ __forceinline__ void park_scales(int srow, uint32_t *ldsSA, uint32_t *ldsSB, int sbuf,
+                                            const uint32_t (&d)[4]) {
+    uint32_t t[4];
+    transpose4x4(d, t);
+    if (srow < S::BM) {
+        uint32_t *dst = ldsSA + sbuf * 4 * S::PA + srow;
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) dst[gg * S::PA] = t[gg];
+    } else {
+        uint32_t *dst = ldsSB + sbuf * 4 * S::PB + (srow - S::BM);
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++) dst[gg * S::PB] = t[gg];
+    }
+}
+
+// One K stage of the workgroup tile: this wave's MT x NT accumulators advance by 128 of K,
+// and, woven between the MFMAs, the wave issues its share of the direct-to-LDS copies that
+// fetch stage `kt_next` (of the tile described by `c`) into LDS buffer `buf_next`.
+//
+// The copies are spread over the first half of the stage on purpose.  The texture path takes
+// 64 bytes per clock, so the 64 KB a stage needs occupy it for ~1000 clocks per CU; issued in
+// one burst at the top of the stage they stall every wave (and the MFMA pipe) for that long,
+// issued late they would not land before the stage-ending barrier.
+template <typename S, int OPSEL>
+__device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, const uint8_t *__restrict__ lb, int a_lo,
+                                              int a_hi, int b_lo, int b_hi, const int (&sa)[S::MT],
+                                              const int (&sb)[S::NT], v4f (&acc)[S::MT][S::NT],
+                                              const IssueCtx<S> &c, const Lane &L, int kt_next, uint8_t *ldsA,
+                                              uint8_t *ldsB, int buf_next) {
+    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt_next * 128);
+    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt_next * 128);
+    const uint32_t wa = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf_next * S::DATA_A + L.wave * 1024);
+    const uint32_t wb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf_next * S::DATA_B + L.wave * 1024);
+    constexpr int NQ = S::QA + S::QB;                      // copies this wave issues per stage
+    constexpr int ISSUE_STEPS = S::MT / 2 > 0 ? S::MT / 2 : 1;  // ... during the first half of the stage
+    auto issue = [&](int q) {
+        if (q < S::QA) dma16(ga, c.a_voff[q], wa + q * S::NW * 1024);
+        else dma16(gb, c.b_voff[q - S::QA], wb + (q - S::QA) * S::NW * 1024);
+    };
+
+    // Nothing crosses into or out of the stage body, nor from one step of it into the next.
+    __builtin_amdgcn_sched_barrier(0);
+    v8i bf[S::NT];
+#pragma unroll
+    for (int j = 0; j < S::NT; j++) {
+        const int o = b_sub_off(j) * 128;
+        v4i lo = *(const v4i *)(lb + b_lo + o);
+        v4i hi = *(const v4i *)(lb + b_hi + o);
+        bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    // A fragments are double buffered in registers: the reads for sub-tile i+1 are in
+    // flight while the MFMAs of sub-tile i issue.
+    v8i af[2];
+    {
+        v4i lo = *(const v4i *)(la + a_lo);
+        v4i hi = *(const v4i *)(la + a_hi);
+        af[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < S::MT; i++) {
+        if (i + 1 < S::MT) {
+            v4i lo = *(const v4i *)(la + a_lo + (i + 1) * (16 * 128));
+            v4i hi = *(const v4i *)(la + a_hi + (i + 1) * (16 * 128));
+            af[(i + 1) & 1] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+        if (i < ISSUE_STEPS) {
+#pragma unroll
+            for (int q = i * NQ / ISSUE_STEPS; q < (i + 1) * NQ / ISSUE_STEPS; q++) issue(q);
+        }
+#pragma unroll
+        for (int j = 0; j < S::NT; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i & 1], acc[i][j], 0, 0, OPSEL,
+                                                                         sb[j], OPSEL, sa[i]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // The MFMAs have no side effects the compiler can see, so it would sink them past the
+    // barrier that ends the stage; an empty volatile asm reading and writing every accumulator
+    // pins them here.
+#pragma unroll
+    for (int i = 0; i < S::MT; i++)
+#pragma unroll
+        for (int j = 0; j < S::NT; j++) asm volatile("" : "+v"(acc[i][j]));
+}
+
+// s_waitcnt with lgkmcnt(0), no expcnt wait, and at most `n` vector-memory operations left in
+// flight (n <= 63).  Vector-memory operations retire in issue order, so this waits for
+// everything except the youngest n.
+__device__ __forceinline__ void wait_vm_allow(int n) {
+    // simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
+    switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0070); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0071); break;
+    default: break;
+    }
+}
+template <int N>
+__device__ __forceinline__ void wait_vm_allow_c() {
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(((N & 15) | (7 << 4) | ((N >> 4) << 14)));
+}
+
+// The persistent tile loop.  `P` (the problem policy) provides
+//   bool P::next(Tile &t)                   advance to this workgroup's next tile (false = done);
+//                                           tiles with an empty K range are finished inside next()
+//   void P::context(const Tile &, const Lane &, IssueCtx<S> &)
+//   const uint8_t *P::line(const Tile &, int operand_row)   address of K byte 0 of row
+//                                           operand_row of the [A rows; B rows] list (for L2 touches)
+//   int  P::epilogue(const Tile &, const Lane &, v4f (&acc)[MT][NT])   returns how many stores each
+//                                           lane issued if that number is the same compile-time
+//                                           constant P::NST for the whole wave, else -1
+//   int  P::kb_end                          scale bytes per row (bound for predicated fetches)
+template <typename S, bool K512, typename P>
+__device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
+    uint8_t *const ldsA = smem;                                                  // [2][BM*128]
+    uint8_t *const ldsB = smem + 2 * S::DATA_A;                                  // [2][BN*128]
+    uint32_t *const ldsSA = (uint32_t *)(smem + 2 * (S::DATA_A + S::DATA_B));    // [2][4][PA]
+    uint32_t *const ldsSB = ldsSA + 2 * 4 * S::PA;                               // [2][4][PB]
+    uint8_t *const ldsJunk = (uint8_t *)(ldsSB + 2 * 4 * S::PB);                 // [NW][256]
+
+    const Lane L = lane_of<S>();
+    const bool has_row0 = L.tid < S::BM + S::BN;
+    const int kb_end = prob.kb_end;
+    constexpr int AHEAD = MX_L2_AHEAD;  // L2 touches run this many stages ahead of the copy engine (0 = off)
+
+    // per-lane LDS read offsets: low half = 16-byte chunk g, high half = chunk g + 4 (= offset ^ 64)
+    const int a_row = L.wm * S::WTM + L.r16;
+    const int b_row = b_tile_row<S>(L.wn, 0, L.r16);
+    const int a_rd = a_row * 128 + ((L.g ^ swz_a(a_row)) << 4);
+    const int b_rd = b_row * 128 + ((L.g ^ swz_b(b_row)) << 4);
+
+    typename P::Tile cur, nxt;
+    if (!prob.next(cur)) return;
+    bool has_next = prob.next(nxt);
+    IssueCtx<S> ctx;
+    prob.context(cur, L, ctx);
+
+    // Lines of stage `k` (relative to the current tile's first stage) that this wave touches:
+    // row tid of the [A rows; B rows] list.  Stages past the tile's end belong to the next tile.
+    auto touch = [&](int k, int KT) -> bool {
+        // every wave issues it (threads past the row list repeat the last row): the stage-end
+        // wait counts on exactly one operation younger than the stage's copies
+        const int r = L.tid < S::BM + S::BN ? L.tid : S::BM + S::BN - 1;
+        const uint8_t *g;
+        if (k < KT) g = prob.line(cur, r) + (int64_t)(cur.kt0 + k) * 128;
+        else if (has_next && k - KT < nxt.kt1 - nxt.kt0) g = prob.line(nxt, r) + (int64_t)(nxt.kt0 + k - KT) * 128;
+        else return false;
+        l2_touch(g, __builtin_amdgcn_readfirstlane(lds_addr(ldsJunk) + L.wave * 256));
+        return true;
+    };
+
+    int gstage = 0;  // stages issued so far, over all tiles: LDS data buffer = gstage & 1
+    int gsuper = 0;  // super-steps so far: LDS scale buffer = gsuper & 1
+
+    // prologue of the first tile
+    {
+        uint32_t d0[4], d1[4];
+        if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);
+        if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);
+        issue_stage<S>(ctx, L, ctx.kt0, ldsA, ldsB, 0);
+        for (int k = 1; k <= AHEAD; k++) touch(k, ctx.kt1 - ctx.kt0);
+        if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
+        if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
+    }
+    wait_vm_allow(0);
+    __syncthreads();
+
+    v4f acc[S::MT][S::NT];
+    while (true) {
+#pragma unroll
+        for (int i = 0; i < S::MT; i++)
+#pragma unroll
+            for (int j = 0; j < S::NT; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+        const int kt0 = ctx.kt0, KT = ctx.kt1 - ctx.kt0;
+        const int nsuper = (KT + 3) >> 2;
+        uint32_t d0[4], d1[4];  // scale bytes in flight: next super-step's, or the next tile's first
+        for (int ss = 0; ss < nsuper; ss++) {
+            const int sbuf = gsuper & 1;
+            int sa[S::MT], sb[S::NT];
+#pragma unroll
+            for (int i = 0; i < S::MT; i++) sa[i] = (int)ldsSA[(sbuf * 4 + L.g) * S::PA + a_row + 16 * i];
+#pragma unroll
+            for (int j = 0; j < S::NT; j++)
+                sb[j] = (int)ldsSB[(sbuf * 4 + L.g) * S::PB + b_row + b_sub_off(j)];
+
+            // One K stage.  In every stage but the tile's last, the next stage's operands are
+            // put in flight first, then the L2 touch for the stage AHEAD beyond it, which is the
+            // only vector-memory operation allowed to stay in flight across the stage's end.
+            // In the last stage nothing of this tile is left to fetch, so the copy context is
+            // switched to the next tile and ITS first stage and scales go in flight; the wait
+            // and barrier that publish them come after the epilogue.
+#define MX_STAGE(SIDX)                                                                                        \
+    {                                                                                                         \
+        const int k = ss * 4 + SIDX;                                                                          \
+        if (k < KT) {                                                                                         \
+            const int buf = gstage & 1;                                                                       \
+            const bool last = k + 1 == KT;                                                                    \
+            bool touched = false;                                                                             \
+            int kt_issue = kt0 + k + 1;                                                                       \
+            if (!last) {                                                                                      \
+                if (SIDX == 3) {                                                                              \
+                    if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, sbuf ^ 1, d0);                          \
+                    if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, sbuf ^ 1, d1);             \
+                }                                                                                             \
+                if (SIDX == 0 && ss + 1 < nsuper) {                                                           \
+                    if (has_row0) load_scales<K512>(ctx.srow0, (kt0 + (ss + 1) * 4) * 4, kb_end, d0);         \
+                    if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, (kt0 + (ss + 1) * 4) * 4, kb_end, d1);      \
+                }                                                                                             \
+            } else if (has_next) {                                                                            \
+                prob.context(nxt, L, ctx);                                                                    \
+                if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);                          \
+                if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);                       \
+                kt_issue = ctx.kt0;                                                                           \
+            } else {                                                                                          \
+                kt_issue = kt0 + k; /* nothing left to fetch: a harmless re-read of this stage */             \
+            }                                                                                                 \
+            compute_stage<S, SIDX>(ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64, b_rd,     \
+                                   b_rd ^ 64, sa, sb, acc, ctx, L, kt_issue, ldsA, ldsB, buf ^ 1);            \
+            if (!last) {                                                                                      \
+                touched = AHEAD && touch(k + 1 + AHEAD, KT);                                                  \
+                if (touched) wait_vm_allow(1);                                                                \
+                else wait_vm_allow(0);                                                                        \
+                __syncthreads();                                                                              \
+            }                                                                                                 \
+            gstage++;                                                                                         \
+        }                                                                                                     \
+    }
+            MX_STAGE(0)
+            MX_STAGE(1)
+            MX_STAGE(2)
+            MX_STAGE(3)
+#undef MX_STAGE
+            gsuper++;
+        }
+        // The next tile's first stage and scales are already in flight: the epilogue's
+        // conversions run under that latency, and when every lane issued the same known number
+        // of stores the wait lets exactly those (and the L2 touch before them) stay in flight,
+        // so the stores drain under the next tile's first stage.
+        const int stores = prob.epilogue(cur, L, acc);
+        if (has_next) {
+            if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
+            if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);
+        }
+        if (!has_next) break;
+        const bool touched = AHEAD && stores == P::NST && touch(KT + AHEAD, KT);
+        if (stores == P::NST && touched) wait_vm_allow_c<P::NST + 1>();
+        else if (stores == P::NST) wait_vm_allow_c<P::NST>();
+        else wait_vm_allow(0);
+        __syncthreads();
+        cur = nxt;
+        has_next = prob.next(nxt);
+    }
+}
+
+// Converts 8 consecutive-N accumulator values of one output row and stores them (one 16-byte
+// store for 16-bit outputs when `vec`).
+template <int CDT>
+__device__ __forceinline__ void store8(void *c, int64_t off, const v4f &lo, const v4f &hi, int nvalid, bool vec) {
+    const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (CDT == MX_FP32) {
+        float *p = (float *)c + off;
+        if (vec && nvalid >= 8) {
+            ((v4f *)p)[0] = lo;
+            ((v4f *)p)[1] = hi;
+        } else {
+            for (int i = 0; i < 8 && i < nvalid; i++) p[i] = v[i];
+        }
+    } else {
+        uint32_t w[4];
+        if (CDT == MX_BF16) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) w[i] = pack2_bf16(v[2 * i], v[2 * i + 1]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                h2 h = {(_Float16)v[2 * i], (_Float16)v[2 * i + 1]};
+                w[i] = __builtin_bit_cast(uint32_t, h);
+            }
+        }
+        uint16_t *p = (uint16_t *)c + off;
+        if (vec && nvalid >= 8) {
+            *(v4i *)p = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        } else {
+            for (int i = 0; i < 8 && i < nvalid; i++) p[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
+        }
+    }
+}
+
+// Maps a flat tile id to (tile_m, tile_n) so that (a) ids congruent mod 8 -- which run on the
+// same XCD, since workgroups are dealt to the 8 XCDs round-robin and the persistent stride is
+// a multiple of 8 -- are neighbours in tile space and share A/B panels in that XCD's L2, and
+// (b) tiles are walked in column groups of GROUP_M row tiles.
+__device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &tm, int &tn) {
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = total >> 3;
+    if (id < (per_xcd << 3)) id = (id & 7) * per_xcd + (id >> 3);
+    constexpr int GROUP_M = 8;
+    const int width = GROUP_M * tiles_n;
+    const int group = id / width;
+    const int first = group * GROUP_M;
+    const int rows = tiles_m - first < GROUP_M ? tiles_m - first : GROUP_M;
+    const int in = id - group * width;
+    tm = first + in % rows;
+    tn = in / rows;
+}
+
+}  // namespace mx

@@ -88,6 +88,26 @@ def test_gemm_exact_integers(oracle):
     assert torch.equal(got.double(), ref)
 
 
+def test_gemm_16bit_rounding_is_nearest_even(oracle):
+    """Exact integer sums, so the only rounding is the output cast: it must equal torch's RTNE cast bit for bit."""
+    m, n, k = 256, 256, 512
+    g = torch.Generator().manual_seed(SEED)
+    codes = torch.tensor([0x30, 0x38, 0x40, 0x44, 0x48, 0xB8, 0xC0], dtype=torch.uint8)  # .5 1 2 3 4 -1 -2
+    aq = codes[torch.randint(0, 7, (m, k), generator=g)]
+    bq = codes[torch.randint(0, 7, (n, k), generator=g)]
+    as_ = torch.randint(127, 131, (m, k // 32), generator=g).to(torch.uint8)
+    bs = torch.randint(127, 131, (n, k // 32), generator=g).to(torch.uint8)
+    exact = oracle.gemm_nt(aq, as_, bq, bs)
+    assert torch.equal(exact, exact.float().double())  # representable in fp32: no accumulation rounding
+    for dtype in (torch.bfloat16, torch.float16):
+        got = _run(aq, as_, bq, bs, dtype)
+        ref = exact.float().to(dtype)
+        if dtype == torch.float16:
+            keep = exact.abs() < 60000
+            got, ref = got[keep], ref[keep]
+        assert torch.equal(got, ref), dtype
+
+
 def test_gemm_scale_extremes(oracle):
     """Scale bytes across the range the quantizer can emit (19..247), products kept finite."""
     m, n, k = 64, 64, 256
