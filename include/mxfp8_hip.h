@@ -130,6 +130,93 @@ int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const ui
                int64_t lda, int64_t ldas, int64_t ldb, int64_t ldbs, int64_t ldc,
                int epilogue, void *stream);
 
+/*
+ * ---- routed experts -------------------------------------------------------------------
+ * Rows are sorted by expert.  `offsets` (E+1) int32 lives on the DEVICE (exclusive prefix sum
+ * of per-expert row counts, truncated to the real experts) and is never read on the host: the
+ * launch is bounded from M and E alone, so a layer stays graph-capturable
+ * (src/kohakuwullm/kernels/mxfp8/grouped.py:3-4,274-275).  Rows outside every expert's range
+ * are not written.  Expert weights: codes (E,NB,K) with strides (stride_we, ldw) and scales
+ * (E,NB,K/32) with strides (stride_wse, ldws).
+ */
+
+/*
+ * out[m] = xq[index[m] or m] . wq[e(m)]^T for sorted positions m < offsets[E]; out (M,N).
+ * xq has a_rows rows.  Replaces grouped_mxfp8_gemm / _grouped_mxfp8_fwd / tile_owner
+ * (src/kohakuwullm/kernels/mxfp8/grouped.py:26-48,65-149,254-327).
+ */
+int mx_grouped_gemm_nt(const uint8_t *xq, const uint8_t *xs, int64_t a_rows, int64_t ldx, int64_t ldxs,
+                       const int32_t *index, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
+                       int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                       void *out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K, void *stream);
+
+/*
+ * Expert GEMM1 with its epilogue: rows gathered by token_of, both halves of x . w_in^T
+ * (w_in (E,2H,K), gate rows first), accumulators rounded to act_dtype, optional store of
+ * pre (M,2H), h = gate * sigmoid(gate) * value quantized per 32 of H into hq (M,H), hs (M,H/32).
+ * Replaces _experts_gemm1 / launch_gemm1 (src/kohakuwullm/kernels/mxfp8/experts.py:25-135,225-275).
+ */
+int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T, int64_t ldx, int64_t ldxs,
+                     const int32_t *token_of, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
+                     int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                     uint8_t *hq, int64_t ldhq, uint8_t *hs, int64_t ldhs, void *pre, int64_t ldpre,
+                     int act_dtype, int64_t M, int64_t H, int64_t K, void *stream);
+
+/*
+ * out[token_of[m]] += scale(m) * (aq[index[m] or m] . wq[e(m)]^T) with packed 16-bit atomic
+ * adds into a caller-zeroed out (T,N); scale(m) = gate[order[m]] when gate != NULL, else 1.
+ * With a gate: _experts_gemm2 / launch_gemm2 (experts.py:138-222,278-323).  Without: the
+ * GEMM1 dgrad _experts_gemm1_dgrad (src/kohakuwullm/kernels/mxfp8/experts_bwd.py:167-247).
+ */
+int mx_experts_scatter_gemm(const uint8_t *aq, const uint8_t *as, int64_t a_rows, int64_t lda, int64_t ldas,
+                            const int32_t *index, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
+                            int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                            const int32_t *token_of, const int32_t *order, const void *gate, int gate_dtype,
+                            void *out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K, void *stream);
+
+/*
+ * DGRAD through GEMM2, the combine and SwiGLU at once: acc = dq[token_of[m]] . w_out_dgrad[e]^T
+ * (M,H); dgate[order[m]] += <acc, dequant(hq,hs)[m]> (fp32 atomics, caller-zeroed);
+ * dh = acc * gate[order[m]]; SwiGLU backward from the stored pre; dpre (M,2H) stored in
+ * act_dtype and quantized from the fp32 values into dpq (M,2H), dps (M,2H/32).
+ * Replaces _experts_gemm2_dgrad (src/kohakuwullm/kernels/mxfp8/experts_bwd.py:29-164).
+ */
+int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int64_t T, int64_t lddq, int64_t ldds,
+                           const int32_t *token_of, const int32_t *order, const void *gate, int gate_dtype,
+                           const uint8_t *wq, const uint8_t *ws, int64_t stride_we, int64_t ldw,
+                           int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                           const uint8_t *hq, int64_t ldhq, const uint8_t *hs, int64_t ldhs, const void *pre,
+                           void *dpre, int64_t ldpre, uint8_t *dpq, int64_t lddpq, uint8_t *dps, int64_t lddps,
+                           float *dgate, int act_dtype, int64_t M, int64_t H, int64_t K, void *stream);
+
+/*
+ * Token-axis quantizer over expert-sorted rows, feeding the experts' MXFP8 WGRAD.  Each
+ * expert's rows are laid out from a fresh multiple of 128 in a padded position space of
+ * Mpad = (ceil(M/128) + E) * 128 positions (rows past an expert's end are zero), so no 32-row
+ * block straddles two experts.  Output qT (C,Mpad), sT (C,Mpad/32).
+ * source 0: x[index[m] or m][0:C], optionally times row_scale[scale_index[m] or m] in fp32 --
+ *           the gathered, gate-scaled dout rows and the gathered x rows of
+ *           grouped_mxfp8_wgrad_kernel (src/kohakuwullm/kernels/mxfp8/grouped.py:152-247);
+ * source 1: silu(x[m][c]) * x[m][C + c] from the stored pre-activation (M,2C) -- the h the
+ *           reference rebuilds in src/kohakuwullm/kernels/mxfp8/moe.py:288-290.
+ */
+int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, int64_t C, int source,
+                             const int32_t *index, const void *row_scale, int row_scale_dtype,
+                             const int32_t *scale_index, const int32_t *offsets, int64_t E, int64_t M,
+                             uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
+
+/*
+ * dW[e] (N,Kout) = AT[:, seg(e)] . BT[:, seg(e)]^T over the padded positions expert e owns,
+ * AT (N,Mpad), BT (Kout,Mpad) from mx_quantize_cols_grouped; dW (E,N,Kout) with strides
+ * (stride_dwe, lddw) in elements.  An expert without rows gets zeros.  The MXFP8 form of
+ * grouped_mxfp8_wgrad_kernel / _launch_wgrad (grouped.py:152-247, moe.py:64-99), which
+ * multiply in 16 bits.
+ */
+int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t lda, int64_t ldas, const uint8_t *bq,
+                        const uint8_t *bs, int64_t ldb, int64_t ldbs, const int32_t *offsets, int64_t E,
+                        int64_t M, void *dw, int dw_dtype, int64_t stride_dwe, int64_t lddw, int64_t N,
+                        int64_t Kout, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

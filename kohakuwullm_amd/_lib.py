@@ -34,6 +34,21 @@ SIGNATURES = {
     "mx_swiglu_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
     "mx_swiglu_bwd_quantize_dual": (
         _ci, [_p, _i64, _p, _i64, _ci, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_grouped_gemm_nt": (
+        _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p]),
+    "mx_experts_gemm1": (
+        _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64,
+              _ci, _i64, _i64, _i64, _p]),
+    "mx_experts_scatter_gemm": (
+        _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _ci, _p, _ci, _i64,
+              _i64, _i64, _i64, _p]),
+    "mx_experts_gemm2_dgrad": (
+        _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _ci, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64,
+              _p, _p, _i64, _p, _i64, _p, _i64, _p, _ci, _i64, _i64, _i64, _p]),
+    "mx_quantize_cols_grouped": (
+        _ci, [_p, _ci, _i64, _i64, _ci, _p, _p, _ci, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_grouped_wgrad_nt": (
+        _ci, [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p]),
     "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),
 }
 

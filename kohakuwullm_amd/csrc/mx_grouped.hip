@@ -1,0 +1,772 @@
+// Routed-expert (grouped) MXFP8 GEMMs for gfx950.
+//
+// Rows are sorted by expert; `offsets (E+1)` int32 on the DEVICE is the exclusive prefix sum
+// of the per-expert row counts and is never read on the host: the grid is a bound
+// (ceil(M/BM) + E row tiles) and every workgroup resolves its row tile to (expert, start, end)
+// itself, as tile_owner does in the reference (src/kohakuwullm/kernels/mxfp8/grouped.py:26-48).
+// Empty experts contribute no tiles; row tiles past the last real one are skipped.
+//
+// One kernel body (mx_gemm_core.h) serves four problems, selected by the policy's MODE:
+//   PLAIN      out[m] = xq[index[m] or m] . wq[e(m)]^T                    grouped.py:65-149
+//   GEMM1      gather by token, both halves of x . w_in^T, round to the storage dtype, SwiGLU,
+//              requantize: hq (M,H), hs (M,H/32), optional pre (M,2H)     experts.py:25-135
+//   SCATTER    out[token(m)] += scale(m) * (a[m] . w[e(m)]^T), packed 16-bit atomics;
+//              scale = gate[order[m]] (GEMM2, experts.py:138-222) or 1 (GEMM1 dgrad,
+//              experts_bwd.py:167-247)
+//   DGRAD2     acc = dq[token(m)] . w_out_dgrad[e]^T; dgate[pair] += <acc, h>; dh = acc * gate;
+//              SwiGLU' from the stored pre; dpre (M,2H) stored and requantized
+//                                                                         experts_bwd.py:29-164
+// The row gather costs nothing: every lane of the copy engine supplies its own global address.
+#include "mx_gemm_core.h"
+
+namespace mx {
+
+enum { MODE_PLAIN = 0, MODE_GEMM1 = 1, MODE_SCATTER = 2, MODE_DGRAD2 = 3 };
+
+struct GroupedArgs {
+    // A operand: rows (R,K) + scales, optionally gathered through index[sorted position]
+    const uint8_t *xq, *xs;
+    int64_t ldx, ldxs;
+    const int32_t *index;
+    // B operand: per-expert (E, NB, K) codes + scales
+    const uint8_t *wq, *ws;
+    int64_t stride_we, ldw, stride_wse, ldws;
+    const int32_t *offsets;
+    int E, M, N, K;  // M: bound on sorted rows; N: output width (hidden units H for GEMM1/DGRAD2)
+    int tiles_n, tbound;
+    // outputs / side inputs
+    void *out;  // PLAIN: (M,N); SCATTER: (T,N) accumulated
+    int64_t ldo;
+    int out_vec;
+    const int32_t *token_of, *order;
+    const void *gate;  // (pairs,) in the 16-bit activation dtype or fp32 (gate_f32)
+    int gate_f32;
+    uint8_t *hq, *hs;  // GEMM1 out / DGRAD2 in: (M,H), (M,H/32)
+    int64_t ldhq, ldhs;
+    void *pre;  // GEMM1 out (optional) / DGRAD2 in: (M,2H) 16-bit
+    int64_t ldpre;
+    void *dpre;  // DGRAD2 out: (M,2H) 16-bit
+    uint8_t *dpq, *dps;  // DGRAD2 out: (M,2H), (M,2H/32)
+    int64_t lddpq, lddps;
+    float *dgate;  // DGRAD2 out: (pairs,) fp32, accumulated
+};
+
+template <int CDT>
+__device__ __forceinline__ float load_act(const void *p, int64_t i) {
+    if (CDT == MX_BF16) return bits2f((uint32_t)((const uint16_t *)p)[i] << 16);
+    if (CDT == MX_FP16) return (float)((const _Float16 *)p)[i];
+    return ((const float *)p)[i];
+}
+
+// Round to the 16-bit storage dtype and come back: what the next consumer will read.
+template <int CDT>
+__device__ __forceinline__ void round_pair(float &a, float &b, uint32_t &packed) {
+    if (CDT == MX_BF16) {
+        packed = pack2_bf16(a, b);
+        a = bits2f(packed << 16);
+        b = bits2f(packed & 0xFFFF0000u);
+    } else {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 h = {(_Float16)a, (_Float16)b};
+        packed = __builtin_bit_cast(uint32_t, h);
+        a = (float)h[0];
+        b = (float)h[1];
+    }
+}
+
+template <int CDT>
+__device__ __forceinline__ void unpack8(const v4i &w, float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (CDT == MX_BF16) {
+            v[2 * i] = bits2f((uint32_t)w[i] << 16);
+            v[2 * i + 1] = bits2f((uint32_t)w[i] & 0xFFFF0000u);
+        } else {
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+            h2 h = __builtin_bit_cast(h2, w[i]);
+            v[2 * i] = (float)h[0];
+            v[2 * i + 1] = (float)h[1];
+        }
+    }
+}
+
+template <int CDT>
+__device__ __forceinline__ void atomic_add2(void *base, int64_t off, float a, float b) {
+    if (CDT == MX_BF16) {
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        f2 v = {a, b};
+        __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) b2 *)((uint16_t *)base + off),
+                                                   __builtin_convertvector(v, b2));
+    } else if (CDT == MX_FP16) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v = {(_Float16)a, (_Float16)b};
+        __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) h2 *)((_Float16 *)base + off), v);
+    } else {
+        atomicAdd((float *)base + off, a);
+        atomicAdd((float *)base + off + 1, b);
+    }
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return __fdividef(1.0f, 1.0f + __expf(-x)); }
+
+// max over the four lanes that share an output row (l, l^16, l^32, l^48)
+__device__ __forceinline__ float row_group_max(float a) {
+    a = fmaxf(a, __shfl_xor(a, 16, 64));
+    return fmaxf(a, __shfl_xor(a, 32, 64));
+}
+__device__ __forceinline__ float row_group_sum(float a) {
+    a += __shfl_xor(a, 16, 64);
+    return a + __shfl_xor(a, 32, 64);
+}
+
+template <typename S, int MODE, int CDT>
+struct GroupedProblem {
+    struct Tile {
+        int n0, row0, end, expert, kt0, kt1;
+    };
+    const GroupedArgs p;  // a copy: fields live in scalar registers
+    int next_id;
+    int kb_end;
+    // incremental tile_owner: experts [0, scan_e) own row tiles [0, scan_tiles)
+    int scan_e, scan_tiles;
+
+    // GEMM1 packs 32 gate + 32 value rows of w_in into each wave's 64-row slice of the B tile,
+    // so a tile spans BN/2 hidden units.
+    static constexpr int N_PER_TILE = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
+    static constexpr int NST = S::MT * (S::NT / 2) * (CDT == MX_FP32 ? 2 : 1);
+
+    __device__ GroupedProblem(const GroupedArgs &a)
+        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0) {}
+
+    __device__ __forceinline__ bool next(Tile &t) {
+        const int total = p.tiles_n * p.tbound;
+        const int per_xcd = total >> 3;
+        while (next_id < total) {
+            int id = next_id;
+            next_id += gridDim.x;
+            // ids congruent mod 8 run on one XCD: give each XCD a contiguous range so the
+            // N tiles of one row tile (same A rows, same expert weights) share an L2
+            if (id < (per_xcd << 3)) id = (id & 7) * per_xcd + (id >> 3);
+            const int rt = id / p.tiles_n;
+            const int tn = id - rt * p.tiles_n;
+            if (rt < scan_tiles) {  // ids are monotonic per workgroup except across the XCD remap edge
+                scan_e = 0;
+                scan_tiles = 0;
+            }
+            int e = scan_e, before = scan_tiles, start = 0, end = 0;
+            bool found = false;
+            while (e < p.E) {
+                start = p.offsets[e];
+                end = p.offsets[e + 1];
+                const int tiles = (end - start + S::BM - 1) / S::BM;
+                if (rt < before + tiles) {
+                    found = true;
+                    break;
+                }
+                before += tiles;
+                e++;
+            }
+            scan_e = e;
+            scan_tiles = before;
+            if (!found) continue;  // past the last real row tile
+            t.expert = e;
+            t.row0 = start + (rt - before) * S::BM;
+            t.end = end;
+            t.n0 = tn * N_PER_TILE;
+            t.kt0 = 0;
+            t.kt1 = p.K >> 7;
+            return true;
+        }
+        return false;
+    }
+
+    // source row of the A operand for tile row r (rows past the expert's end repeat its last row)
+    __device__ __forceinline__ int a_src_row(const Tile &t, int r) const {
+        int pos = t.row0 + r;
+        pos = pos < t.end ? pos : t.end - 1;
+        return p.index ? p.index[pos] : pos;
+    }
+    // row of the expert's weight matrix behind B tile row r
+    __device__ __forceinline__ int b_src_row(const Tile &t, int r) const {
+        if (MODE == MODE_GEMM1) {
+            const int slice = r >> 6, within = r & 63;
+            int h = t.n0 + slice * 32 + (within & 31);
+            h = h < p.N ? h : p.N - 1;
+            return within < 32 ? h : p.N + h;
+        }
+        const int n = t.n0 + r;
+        return n < p.N ? n : p.N - 1;
+    }
+
+    __device__ __forceinline__ void context(const Tile &t, const Lane &L0, IssueCtx<S> &c) const {
+        const Lane L = opaque(L0);
+        c.a_base = p.xq;
+        c.b_base = p.wq + (int64_t)t.expert * p.stride_we;
+        c.kt0 = t.kt0;
+        c.kt1 = t.kt1;
+#pragma unroll
+        for (int q = 0; q < S::QA; q++) {
+            const int row = dma_row<S>(L, q);
+            c.a_voff[q] = (uint32_t)((int64_t)a_src_row(t, row) * p.ldx) + (((L.lane & 7) ^ swz_a(row)) << 4);
+        }
+#pragma unroll
+        for (int q = 0; q < S::QB; q++) {
+            const int row = dma_row<S>(L, q);
+            c.b_voff[q] = (uint32_t)((int64_t)b_src_row(t, row) * p.ldw) + (((L.lane & 7) ^ swz_b(row)) << 4);
+        }
+        auto srow = [&](int r) -> const uint8_t * {
+            if (r < S::BM) return p.xs + (int64_t)a_src_row(t, r) * p.ldxs;
+            return p.ws + (int64_t)t.expert * p.stride_wse + (int64_t)b_src_row(t, r - S::BM) * p.ldws;
+        };
+        c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
+        c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
+    }
+
+    __device__ __forceinline__ const uint8_t *line(const Tile &t, int r) const {
+        if (r < S::BM) return p.xq + (int64_t)a_src_row(t, r) * p.ldx;
+        return p.wq + (int64_t)t.expert * p.stride_we + (int64_t)b_src_row(t, r - S::BM) * p.ldw;
+    }
+
+    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        if (MODE == MODE_PLAIN) return epilogue_plain(t, L, acc);
+        if (MODE == MODE_GEMM1) return epilogue_gemm1(t, L, acc);
+        if (MODE == MODE_SCATTER) return epilogue_scatter(t, L, acc);
+        return epilogue_dgrad2(t, L, acc);
+    }
+
+    // ---- PLAIN: rows of the expert's range are written, nothing else is touched
+    __device__ __forceinline__ int epilogue_plain(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        const bool interior = t.row0 + S::BM <= t.end && t.n0 + S::BN <= p.N && p.out_vec;
+#pragma unroll
+        for (int i = 0; i < S::MT; i++) {
+            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
+#pragma unroll
+            for (int h = 0; h < S::NT / 2; h++) {
+                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+                const int64_t off = (int64_t)m * p.ldo + n;
+                if (interior) store8<CDT>(p.out, off, acc[i][2 * h], acc[i][2 * h + 1], 8, true);
+                else if (m < t.end && n < p.N)
+                    store8<CDT>(p.out, off, acc[i][2 * h], acc[i][2 * h + 1], p.N - n < 8 ? p.N - n : 8, p.out_vec != 0);
+            }
+        }
+        return interior ? NST : -1;
+    }
+
+    // ---- GEMM1: sub-tiles (4q, 4q+1) are gate, (4q+2, 4q+3) value of the same 8 hidden units
+    __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+#pragma unroll
+        for (int i = 0; i < S::MT; i++) {
+            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
+            const bool row_ok = m < t.end;
+#pragma unroll
+            for (int q = 0; q < S::NT / 4; q++) {
+                // this wave's 32 hidden units of slice (wn, q); the lane owns 8 of them
+                const int hblock = t.n0 + (L.wn * (S::NT / 4) + q) * 32;
+                const int h = hblock + 8 * L.g;
+                const bool ok = row_ok && hblock < p.N;  // H % 32 == 0: a block is in or out
+                float gv[8], vv[8];
+                uint32_t gp[4], vp[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    gv[e] = acc[i][4 * q][e], gv[4 + e] = acc[i][4 * q + 1][e];
+                    vv[e] = acc[i][4 * q + 2][e], vv[4 + e] = acc[i][4 * q + 3][e];
+                }
+                // h is rounded to the storage dtype before the activation, so the backward
+                // differentiates the function the forward evaluated (experts.py:116-119)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    round_pair<CDT>(gv[2 * e], gv[2 * e + 1], gp[e]);
+                    round_pair<CDT>(vv[2 * e], vv[2 * e + 1], vp[e]);
+                }
+                if (ok && p.pre) {
+                    uint16_t *pp = (uint16_t *)p.pre + (int64_t)m * p.ldpre + h;
+                    *(v4i *)pp = v4i{(int)gp[0], (int)gp[1], (int)gp[2], (int)gp[3]};
+                    *(v4i *)(pp + p.N) = v4i{(int)vp[0], (int)vp[1], (int)vp[2], (int)vp[3]};
+                }
+                float a[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) a[e] = gv[e] * sigmoid_f(gv[e]) * vv[e];
+                const float amax = row_group_max(amax8(a));
+                const uint32_t byte = scale_byte(amax);
+                const float inv = inv_scale(byte);
+                if (ok) {
+                    v2i codes;
+                    codes[0] = (int)pack4_e4m3(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv);
+                    codes[1] = (int)pack4_e4m3(a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+                    *(v2i *)(p.hq + (int64_t)m * p.ldhq + h) = codes;
+                    if (L.g == 0) p.hs[(int64_t)m * p.ldhs + (hblock >> 5)] = (uint8_t)byte;
+                }
+            }
+        }
+        return -1;
+    }
+
+    // ---- SCATTER: out[token(m)] += scale(m) * acc, packed 16-bit (or fp32) atomics
+    __device__ __forceinline__ int epilogue_scatter(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+#pragma unroll
+        for (int i = 0; i < S::MT; i++) {
+            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
+            if (m >= t.end) continue;
+            const int target = p.token_of[m];
+            float scale = 1.0f;
+            if (p.gate) scale = p.gate_f32 ? ((const float *)p.gate)[p.order[m]] : load_act<CDT>(p.gate, p.order[m]);
+#pragma unroll
+            for (int h = 0; h < S::NT / 2; h++) {
+                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+                const int64_t off = (int64_t)target * p.ldo + n;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float a = (e < 2 ? acc[i][2 * h][2 * e] : acc[i][2 * h + 1][2 * e - 4]) * scale;
+                    const float b = (e < 2 ? acc[i][2 * h][2 * e + 1] : acc[i][2 * h + 1][2 * e - 3]) * scale;
+                    if (n + 2 * e + 1 < p.N) atomic_add2<CDT>(p.out, off + 2 * e, a, b);
+                    else if (n + 2 * e < p.N) {
+                        // odd tail: a lone element (N % 2 == 1 never happens for 32-multiples, kept for safety)
+                        atomic_add2<CDT>(p.out, off + 2 * e - 1, 0.0f, a);
+                    }
+                }
+            }
+        }
+        return -1;
+    }
+
+    // ---- DGRAD2: the accumulator dout[t] . W_out is consumed three ways in registers
+    __device__ __forceinline__ int epilogue_dgrad2(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        const int H = p.N;
+#pragma unroll
+        for (int i = 0; i < S::MT; i++) {
+            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
+            const bool row_ok = m < t.end;
+            const int mm = row_ok ? m : t.end - 1;
+            const int pair = p.order[mm];
+            const float gate = p.gate_f32 ? ((const float *)p.gate)[pair] : load_act<CDT>(p.gate, pair);
+            float dot = 0.0f;
+#pragma unroll
+            for (int hh = 0; hh < S::NT / 2; hh++) {
+                const int hblock = t.n0 + L.wn * S::WTN + b_sub_off(2 * hh);  // 32 hidden units of the 4 lanes
+                const int h = hblock + 8 * L.g;
+                const bool ok = row_ok && hblock < H;
+                float a[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[e] = acc[i][2 * hh][e], a[4 + e] = acc[i][2 * hh + 1][e];
+                float dg[8], dv[8];
+                if (ok) {
+                    // h read back from its fp8 copy: the forward multiplied those values
+                    const v2i hc = *(const v2i *)(p.hq + (int64_t)mm * p.ldhq + h);
+                    const float hscale = bits2f((uint32_t)p.hs[(int64_t)mm * p.ldhs + (hblock >> 5)] << 23);
+                    float gq[8], vq[8];
+                    const uint16_t *pp = (const uint16_t *)p.pre + (int64_t)mm * p.ldpre + h;
+                    unpack8<CDT>(*(const v4i *)pp, gq);
+                    unpack8<CDT>(*(const v4i *)(pp + H), vq);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        typedef float v2f __attribute__((ext_vector_type(2)));
+                        const int word = hc[e >> 2];
+                        const v2f pairv = (e & 2) ? __builtin_amdgcn_cvt_pk_f32_fp8(word, true)
+                                                  : __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
+                        const float hval = pairv[e & 1] * hscale;
+                        dot += a[e] * hval;
+                        const float dh = a[e] * gate;
+                        const float sg = sigmoid_f(gq[e]);
+                        dg[e] = dh * vq[e] * sg * (1.0f + gq[e] * (1.0f - sg));
+                        dv[e] = dh * gq[e] * sg;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) dg[e] = dv[e] = 0.0f;
+                }
+                // both halves: store dpre in the storage dtype, quantize from the fp32 values
+                const float amax_g = row_group_max(amax8(dg));
+                const float amax_v = row_group_max(amax8(dv));
+                const uint32_t bg = scale_byte(amax_g), bv = scale_byte(amax_v);
+                const float ig = inv_scale(bg), iv = inv_scale(bv);
+                if (ok) {
+                    uint32_t w[4], x[4];
+                    float tg[8], tv[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) tg[e] = dg[e], tv[e] = dv[e];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        round_pair<CDT>(tg[2 * e], tg[2 * e + 1], w[e]);
+                        round_pair<CDT>(tv[2 * e], tv[2 * e + 1], x[e]);
+                    }
+                    uint16_t *dp = (uint16_t *)p.dpre + (int64_t)m * p.ldpre + h;
+                    *(v4i *)dp = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                    *(v4i *)(dp + H) = v4i{(int)x[0], (int)x[1], (int)x[2], (int)x[3]};
+                    v2i cg, cv;
+                    cg[0] = (int)pack4_e4m3(dg[0] * ig, dg[1] * ig, dg[2] * ig, dg[3] * ig);
+                    cg[1] = (int)pack4_e4m3(dg[4] * ig, dg[5] * ig, dg[6] * ig, dg[7] * ig);
+                    cv[0] = (int)pack4_e4m3(dv[0] * iv, dv[1] * iv, dv[2] * iv, dv[3] * iv);
+                    cv[1] = (int)pack4_e4m3(dv[4] * iv, dv[5] * iv, dv[6] * iv, dv[7] * iv);
+                    uint8_t *qp = p.dpq + (int64_t)m * p.lddpq + h;
+                    *(v2i *)qp = cg;
+                    *(v2i *)(qp + H) = cv;
+                    if (L.g == 0) {
+                        uint8_t *sp = p.dps + (int64_t)m * p.lddps + (hblock >> 5);
+                        sp[0] = (uint8_t)bg;
+                        sp[H >> 5] = (uint8_t)bv;
+                    }
+                }
+            }
+            // the dot product over the expert width is split across lanes, waves and N tiles
+            dot = row_group_sum(dot);
+            if (row_ok && L.g == 0) atomicAdd(p.dgate + pair, dot);
+        }
+        return -1;
+    }
+};
+
+template <typename S, int MODE, int CDT, bool K512>
+__global__ __launch_bounds__(S::NTHR) void grouped_kernel(GroupedArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    GroupedProblem<S, MODE, CDT> prob(args);
+    persistent_gemm<S, K512>(prob, smem);
+}
+
+// Slow path for shapes the tiled kernel does not take (PLAIN only): one thread per output element.
+template <int CDT>
+__global__ __launch_bounds__(256) void grouped_generic_kernel(GroupedArgs p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int last = p.offsets[p.E];
+    const int64_t m = idx / p.N, n = idx - m * p.N;
+    if (m >= last || m >= p.M) return;
+    int e = 0;
+    while (e + 1 < p.E && p.offsets[e + 1] <= m) e++;
+    const int64_t src = p.index ? p.index[m] : m;
+    const uint8_t *pa = p.xq + src * p.ldx, *pb = p.wq + e * p.stride_we + n * p.ldw;
+    const uint8_t *sa = p.xs + src * p.ldxs, *sb = p.ws + e * p.stride_wse + n * p.ldws;
+    float acc = 0.0f;
+    for (int kb = 0; kb < p.K / MX_BLOCK; kb++) {
+        float part = 0.0f;
+        for (int i = 0; i < MX_BLOCK; i += 2) {
+            typedef float v2f __attribute__((ext_vector_type(2)));
+            uint32_t wa = pa[kb * MX_BLOCK + i] | ((uint32_t)pa[kb * MX_BLOCK + i + 1] << 8);
+            uint32_t wb = pb[kb * MX_BLOCK + i] | ((uint32_t)pb[kb * MX_BLOCK + i + 1] << 8);
+            v2f fa = __builtin_amdgcn_cvt_pk_f32_fp8((int)wa, false);
+            v2f fb = __builtin_amdgcn_cvt_pk_f32_fp8((int)wb, false);
+            part += fa[0] * fb[0] + fa[1] * fb[1];
+        }
+        acc += ldexpf(part, (int)sa[kb] + (int)sb[kb] - 254);
+    }
+    if (CDT == MX_FP32) ((float *)p.out)[m * p.ldo + n] = acc;
+    else if (CDT == MX_BF16) ((uint16_t *)p.out)[m * p.ldo + n] = (uint16_t)f2bf16(acc);
+    else ((_Float16 *)p.out)[m * p.ldo + n] = (_Float16)acc;
+}
+
+// ---- grouped WGRAD: dW[e] (N,Kout) = AT[:, seg(e)] . BT[:, seg(e)]^T ------------------------------
+// AT (N, Mpad) and BT (Kout, Mpad) are the token-axis quantizations written by
+// mx_quantize_cols_grouped: expert e owns the padded positions of its 128-row tiles, i.e. K
+// stages [tiles_before(e), tiles_before(e) + tiles(e)).  One writer per element; an expert
+// with no rows gets zeros (grouped.py:152-247 of the reference has the same contract).
+struct WgradArgs {
+    const uint8_t *aq, *as, *bq, *bs;
+    int64_t lda, ldas, ldb, ldbs;
+    void *dw;
+    int64_t stride_dwe, lddw;
+    const int32_t *offsets;
+    int E, N, Kout, KB;  // KB: scale bytes per row of the padded space
+    int tiles_m, tiles_n, c_vec;
+};
+
+template <typename S, int CDT>
+struct WgradProblem {
+    struct Tile {
+        int m0, n0, kt0, kt1, expert;
+    };
+    const WgradArgs p;
+    int next_id, kb_end, scan_e, scan_tiles;
+    static constexpr int NST = S::MT * (S::NT / 2) * (CDT == MX_FP32 ? 2 : 1);
+
+    __device__ WgradProblem(const WgradArgs &a) : p(a), next_id(blockIdx.x), kb_end(a.KB), scan_e(0), scan_tiles(0) {}
+
+    __device__ __forceinline__ void zero_tile(const Tile &t) const {
+        // an expert without rows: its dW tile is zeros
+        const int esz = CDT == MX_FP32 ? 4 : 2;
+        for (int idx = threadIdx.x; idx < S::BM * S::BN; idx += S::NTHR) {
+            const int m = t.m0 + idx / S::BN, n = t.n0 + idx % S::BN;
+            if (m < p.N && n < p.Kout) {
+                char *dst = (char *)p.dw + ((int64_t)t.expert * p.stride_dwe + (int64_t)m * p.lddw + n) * esz;
+                if (esz == 4) *(float *)dst = 0.0f;
+                else *(uint16_t *)dst = 0;
+            }
+        }
+    }
+
+    __device__ __forceinline__ bool next(Tile &t) {
+        const int per_e = p.tiles_m * p.tiles_n;
+        while (next_id < per_e * p.E) {
+            const int id = next_id;
+            next_id += gridDim.x;
+            const int e = id / per_e;
+            const int rem = id - e * per_e;
+            // tiles of experts before e (ids, hence e, only grow for one workgroup)
+            while (scan_e < e) {
+                scan_tiles += (p.offsets[scan_e + 1] - p.offsets[scan_e] + 127) / 128;
+                scan_e++;
+            }
+            t.expert = e;
+            t.m0 = (rem / p.tiles_n) * S::BM;
+            t.n0 = (rem % p.tiles_n) * S::BN;
+            t.kt0 = scan_tiles;
+            t.kt1 = scan_tiles + (p.offsets[e + 1] - p.offsets[e] + 127) / 128;
+            if (t.kt0 == t.kt1) {
+                zero_tile(t);
+                continue;
+            }
+            return true;
+        }
+        return false;
+    }
+
+    __device__ __forceinline__ void context(const Tile &t, const Lane &L0, IssueCtx<S> &c) const {
+        const Lane L = opaque(L0);
+        c.a_base = p.aq + (int64_t)t.m0 * p.lda;
+        c.b_base = p.bq + (int64_t)t.n0 * p.ldb;
+        c.kt0 = t.kt0;
+        c.kt1 = t.kt1;
+        const int mrem = p.N - t.m0, nrem = p.Kout - t.n0;
+#pragma unroll
+        for (int q = 0; q < S::QA; q++) {
+            const int row = dma_row<S>(L, q);
+            c.a_voff[q] = (uint32_t)((int64_t)(row < mrem ? row : mrem - 1) * p.lda) + (((L.lane & 7) ^ swz_a(row)) << 4);
+        }
+#pragma unroll
+        for (int q = 0; q < S::QB; q++) {
+            const int row = dma_row<S>(L, q);
+            c.b_voff[q] = (uint32_t)((int64_t)(row < nrem ? row : nrem - 1) * p.ldb) + (((L.lane & 7) ^ swz_b(row)) << 4);
+        }
+        auto srow = [&](int r) -> const uint8_t * {
+            if (r < S::BM) return p.as + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.ldas;
+            r -= S::BM;
+            return p.bs + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldbs;
+        };
+        c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
+        c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
+    }
+
+    __device__ __forceinline__ const uint8_t *line(const Tile &t, int r) const {
+        if (r < S::BM) return p.aq + (int64_t)(t.m0 + r < p.N ? t.m0 + r : p.N - 1) * p.lda;
+        r -= S::BM;
+        return p.bq + (int64_t)(t.n0 + r < p.Kout ? t.n0 + r : p.Kout - 1) * p.ldb;
+    }
+
+    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        const bool interior = t.m0 + S::BM <= p.N && t.n0 + S::BN <= p.Kout && p.c_vec;
+        const int64_t base = (int64_t)t.expert * p.stride_dwe;
+#pragma unroll
+        for (int i = 0; i < S::MT; i++) {
+            const int m = t.m0 + L.wm * S::WTM + 16 * i + L.r16;
+#pragma unroll
+            for (int h = 0; h < S::NT / 2; h++) {
+                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+                const int64_t off = base + (int64_t)m * p.lddw + n;
+                if (interior) store8<CDT>(p.dw, off, acc[i][2 * h], acc[i][2 * h + 1], 8, true);
+                else if (m < p.N && n < p.Kout)
+                    store8<CDT>(p.dw, off, acc[i][2 * h], acc[i][2 * h + 1], p.Kout - n < 8 ? p.Kout - n : 8, p.c_vec != 0);
+            }
+        }
+        return interior ? NST : -1;
+    }
+};
+
+template <typename S, int CDT>
+__global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    WgradProblem<S, CDT> prob(args);
+    persistent_gemm<S, false>(prob, smem);
+}
+
+}  // namespace mx
+
+using namespace mx;
+
+static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+static int num_cus() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    return n;
+}
+
+typedef GemmShape<256, 256, 2, 4> Big;
+
+static bool tiled_ok(const GroupedArgs &a, int64_t a_rows) {
+    return a.K % 128 == 0 && aligned(a.xq, 16) && aligned(a.wq, 16) && a.ldx % 16 == 0 && a.ldw % 16 == 0 &&
+           a.stride_we % 16 == 0 && aligned(a.xs, 4) && aligned(a.ws, 4) && a.ldxs % 4 == 0 && a.ldws % 4 == 0 &&
+           a.stride_wse % 4 == 0 && a_rows * a.ldx < ((int64_t)1 << 32) && (int64_t)a.N * 2 * a.ldw < ((int64_t)1 << 32);
+}
+
+template <int MODE, int CDT>
+static int launch_grouped(GroupedArgs a, hipStream_t st) {
+    typedef Big S;
+    constexpr int npt = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
+    a.tiles_n = (a.N + npt - 1) / npt;
+    a.tbound = (a.M + S::BM - 1) / S::BM + a.E;
+    const int64_t work = (int64_t)a.tiles_n * a.tbound;
+    if (work >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    const bool k512 = a.K % 512 == 0 && aligned(a.xs, 16) && aligned(a.ws, 16) && a.ldxs % 16 == 0 &&
+                      a.ldws % 16 == 0 && a.stride_wse % 16 == 0;
+    const int cus = num_cus();
+    dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
+    auto kern = k512 ? grouped_kernel<S, MODE, CDT, true> : grouped_kernel<S, MODE, CDT, false>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
+        return MX_ELAUNCH;
+    kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+template <int MODE>
+static int launch_grouped_dt(int dt, const GroupedArgs &a, hipStream_t st) {
+    switch (dt) {
+    case MX_BF16: return launch_grouped<MODE, MX_BF16>(a, st);
+    case MX_FP16: return launch_grouped<MODE, MX_FP16>(a, st);
+    default: return MX_EINVAL;
+    }
+}
+
+static GroupedArgs base_args(const uint8_t *xq, const uint8_t *xs, int64_t ldx, int64_t ldxs, const int32_t *index,
+                             const uint8_t *wq, const uint8_t *ws, int64_t stride_we, int64_t ldw, int64_t stride_wse,
+                             int64_t ldws, const int32_t *offsets, int64_t E, int64_t M, int64_t N, int64_t K) {
+    GroupedArgs a = {};
+    a.xq = xq, a.xs = xs, a.ldx = ldx, a.ldxs = ldxs, a.index = index;
+    a.wq = wq, a.ws = ws, a.stride_we = stride_we, a.ldw = ldw, a.stride_wse = stride_wse, a.ldws = ldws;
+    a.offsets = offsets, a.E = (int)E, a.M = (int)M, a.N = (int)N, a.K = (int)K;
+    return a;
+}
+
+static bool sizes_ok(int64_t E, int64_t M, int64_t N, int64_t K) {
+    return E > 0 && E < (1 << 20) && M >= 0 && M < 0x7FFFFFFF && N >= 0 && N < 0x7FFFFFFF && K >= 0 && K < 0x7FFFFFFF &&
+           K % MX_BLOCK == 0;
+}
+
+extern "C" int mx_grouped_gemm_nt(const uint8_t *xq, const uint8_t *xs, int64_t a_rows, int64_t ldx, int64_t ldxs,
+                                  const int32_t *index, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
+                                  int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                                  void *out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K, void *stream) {
+    if (!sizes_ok(E, M, N, K) || ldx < K || ldw < K || ldo < N) return MX_EINVAL;
+    if (M == 0 || N == 0) return MX_OK;
+    hipStream_t st = (hipStream_t)stream;
+    GroupedArgs a = base_args(xq, xs, ldx, ldxs, index, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, N, K);
+    a.out = out, a.ldo = ldo;
+    const int esz = out_dtype == MX_FP32 ? 4 : 2;
+    a.out_vec = aligned(out, 16) && (ldo * esz) % 16 == 0;
+    if (K == 0 || !tiled_ok(a, a_rows)) {
+        if (K == 0) return MX_EUNSUPPORTED;
+        int64_t blocks = (M * N + 255) / 256;
+        if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
+        switch (out_dtype) {
+        case MX_BF16: grouped_generic_kernel<MX_BF16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a); break;
+        case MX_FP16: grouped_generic_kernel<MX_FP16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a); break;
+        case MX_FP32: grouped_generic_kernel<MX_FP32><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a); break;
+        default: return MX_EINVAL;
+        }
+        return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+    }
+    switch (out_dtype) {
+    case MX_BF16: return launch_grouped<MODE_PLAIN, MX_BF16>(a, st);
+    case MX_FP16: return launch_grouped<MODE_PLAIN, MX_FP16>(a, st);
+    case MX_FP32: return launch_grouped<MODE_PLAIN, MX_FP32>(a, st);
+    default: return MX_EINVAL;
+    }
+}
+
+extern "C" int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T, int64_t ldx, int64_t ldxs,
+                                const int32_t *token_of, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
+                                int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                                uint8_t *hq, int64_t ldhq, uint8_t *hs, int64_t ldhs, void *pre, int64_t ldpre,
+                                int act_dtype, int64_t M, int64_t H, int64_t K, void *stream) {
+    if (!sizes_ok(E, M, H, K) || H % MX_BLOCK || ldx < K || ldw < K || ldhq < H || ldhs < H / MX_BLOCK ||
+        (pre && ldpre < 2 * H) || !token_of)
+        return MX_EINVAL;
+    if (M == 0 || H == 0) return MX_OK;
+    GroupedArgs a = base_args(xq, xs, ldx, ldxs, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
+    a.hq = hq, a.ldhq = ldhq, a.hs = hs, a.ldhs = ldhs, a.pre = pre, a.ldpre = ldpre;
+    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 16) || ldpre % 8 || H % 8)))
+        return MX_EUNSUPPORTED;
+    return launch_grouped_dt<MODE_GEMM1>(act_dtype, a, (hipStream_t)stream);
+}
+
+extern "C" int mx_experts_scatter_gemm(const uint8_t *aq, const uint8_t *as, int64_t a_rows, int64_t lda, int64_t ldas,
+                                       const int32_t *index, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
+                                       int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets,
+                                       int64_t E, const int32_t *token_of, const int32_t *order, const void *gate,
+                                       int gate_dtype, void *out, int out_dtype, int64_t ldo, int64_t M, int64_t N,
+                                       int64_t K, void *stream) {
+    if (!sizes_ok(E, M, N, K) || N % 2 || lda < K || ldw < K || ldo < N || !token_of || (gate && !order)) return MX_EINVAL;
+    if (gate && gate_dtype != MX_FP32 && gate_dtype != out_dtype) return MX_EINVAL;
+    if (M == 0 || N == 0) return MX_OK;
+    GroupedArgs a = base_args(aq, as, lda, ldas, index, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, N, K);
+    a.token_of = token_of, a.order = order, a.gate = gate, a.gate_f32 = gate_dtype == MX_FP32;
+    a.out = out, a.ldo = ldo;
+    if (K == 0 || !tiled_ok(a, a_rows) || !aligned(out, 4) || ldo % 2) return MX_EUNSUPPORTED;
+    return launch_grouped_dt<MODE_SCATTER>(out_dtype, a, (hipStream_t)stream);
+}
+
+extern "C" int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int64_t T, int64_t lddq, int64_t ldds,
+                                      const int32_t *token_of, const int32_t *order, const void *gate, int gate_dtype,
+                                      const uint8_t *wq, const uint8_t *ws, int64_t stride_we, int64_t ldw,
+                                      int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
+                                      const uint8_t *hq, int64_t ldhq, const uint8_t *hs, int64_t ldhs, const void *pre,
+                                      void *dpre, int64_t ldpre, uint8_t *dpq, int64_t lddpq, uint8_t *dps,
+                                      int64_t lddps, float *dgate, int act_dtype, int64_t M, int64_t H, int64_t K,
+                                      void *stream) {
+    if (!sizes_ok(E, M, H, K) || H % MX_BLOCK || lddq < K || ldw < K || ldhq < H || ldpre < 2 * H || lddpq < 2 * H ||
+        lddps < 2 * H / MX_BLOCK || !token_of || !order || !gate || !pre || !dpre || !dgate)
+        return MX_EINVAL;
+    if (gate_dtype != MX_FP32 && gate_dtype != act_dtype) return MX_EINVAL;
+    if (M == 0 || H == 0) return MX_OK;
+    GroupedArgs a = base_args(dq, ds, lddq, ldds, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
+    a.token_of = token_of, a.order = order, a.gate = gate, a.gate_f32 = gate_dtype == MX_FP32;
+    a.hq = (uint8_t *)hq, a.ldhq = ldhq, a.hs = (uint8_t *)hs, a.ldhs = ldhs;
+    a.pre = (void *)pre, a.dpre = dpre, a.ldpre = ldpre, a.dpq = dpq, a.lddpq = lddpq, a.dps = dps, a.lddps = lddps;
+    a.dgate = dgate;
+    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || !aligned(pre, 16) || !aligned(dpre, 16) ||
+        ldpre % 8 || H % 8 || !aligned(dpq, 8) || lddpq % 8)
+        return MX_EUNSUPPORTED;
+    return launch_grouped_dt<MODE_DGRAD2>(act_dtype, a, (hipStream_t)stream);
+}
+
+template <int CDT>
+static int launch_wgrad(WgradArgs a, hipStream_t st) {
+    typedef Big S;
+    a.tiles_m = (a.N + S::BM - 1) / S::BM;
+    a.tiles_n = (a.Kout + S::BN - 1) / S::BN;
+    const int esz = CDT == MX_FP32 ? 4 : 2;
+    a.c_vec = aligned(a.dw, 16) && (a.lddw * esz) % 16 == 0 && (a.stride_dwe * esz) % 16 == 0;
+    const int64_t work = (int64_t)a.tiles_m * a.tiles_n * a.E;
+    if (work >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    const int cus = num_cus();
+    dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
+    auto kern = grouped_wgrad_kernel<S, CDT>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
+        return MX_ELAUNCH;
+    kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+extern "C" int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t lda, int64_t ldas, const uint8_t *bq,
+                                   const uint8_t *bs, int64_t ldb, int64_t ldbs, const int32_t *offsets, int64_t E,
+                                   int64_t M, void *dw, int dw_dtype, int64_t stride_dwe, int64_t lddw, int64_t N,
+                                   int64_t Kout, void *stream) {
+    if (E <= 0 || E >= (1 << 20) || M < 0 || M >= 0x7FFFFFFF || N < 0 || Kout < 0 || N >= 0x7FFFFFFF ||
+        Kout >= 0x7FFFFFFF || lddw < Kout)
+        return MX_EINVAL;
+    const int64_t mpad = ((M + 127) / 128 + E) * 128;
+    if (lda < mpad || ldb < mpad || ldas < mpad / MX_BLOCK || ldbs < mpad / MX_BLOCK) return MX_EINVAL;
+    if (N == 0 || Kout == 0) return MX_OK;
+    if (!aligned(aq, 16) || !aligned(bq, 16) || lda % 16 || ldb % 16 || !aligned(as, 4) || !aligned(bs, 4) || ldas % 4 ||
+        ldbs % 4 || 256 * lda >= ((int64_t)1 << 32) || 256 * ldb >= ((int64_t)1 << 32))
+        return MX_EUNSUPPORTED;
+    WgradArgs a = {};
+    a.aq = aq, a.as = as, a.bq = bq, a.bs = bs, a.lda = lda, a.ldas = ldas, a.ldb = ldb, a.ldbs = ldbs;
+    a.dw = dw, a.stride_dwe = stride_dwe, a.lddw = lddw, a.offsets = offsets, a.E = (int)E, a.N = (int)N,
+    a.Kout = (int)Kout, a.KB = (int)(mpad / MX_BLOCK);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dw_dtype) {
+    case MX_BF16: return launch_wgrad<MX_BF16>(a, st);
+    case MX_FP16: return launch_wgrad<MX_FP16>(a, st);
+    case MX_FP32: return launch_wgrad<MX_FP32>(a, st);
+    default: return MX_EINVAL;
+    }
+}

@@ -387,6 +387,85 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows_kernel(const void *__re
     }
 }
 
+// ------------------------------------------------------------------------------------
+// Column-axis quantizer over expert-sorted rows, for the routed experts' MXFP8 WGRAD.
+// WGRAD contracts the rows an expert owns, so the 32-row blocks must not straddle two experts:
+// every expert's segment is laid out from a fresh multiple of 128 in a padded position space
+// (tile t of 128 rows = positions [128 t, 128 t + 128)), rows past the segment's end are zero.
+// Row tile -> (expert, first row) is resolved on the device from `offsets`, like the GEMMs.
+// Sources: SRC_PLAIN  x[index[m] or m] (optionally times row_scale[scale_index[m]] in fp32,
+//                     the gate applied to dout rows: grouped.py:218-221 of the reference)
+//          SRC_SWIGLU silu(pre[m][c]) * pre[m][H + c] in fp32 (moe.py:288-290 rebuilds h from pre)
+// ------------------------------------------------------------------------------------
+
+enum { SRC_PLAIN = 0, SRC_SWIGLU = 1 };
+
+struct GroupedQuantArgs {
+    const void *x;
+    int64_t ldx;
+    int C;  // output columns of x to quantize (H for SRC_SWIGLU, whose x has 2H columns)
+    const int32_t *index;
+    const void *row_scale;
+    const int32_t *scale_index;
+    int scale_f32;
+    const int32_t *offsets;
+    int E;
+};
+
+template <int DT, int SRC>
+__global__ __launch_bounds__(256) void quant_cols_grouped_kernel(GroupedQuantArgs a, QuantTileOut o, int64_t mpad) {
+    typedef typename Elem<DT>::type T;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+    const int t = threadIdx.x;
+    const int rt = blockIdx.y;
+    // tile_owner: experts whose tiles all precede rt
+    int e = 0, before = 0, start = 0, end = 0;
+    bool found = false;
+    for (; e < a.E; e++) {
+        start = a.offsets[e];
+        end = a.offsets[e + 1];
+        const int tiles = (end - start + QC_TILE - 1) / QC_TILE;
+        if (rt < before + tiles) {
+            found = true;
+            break;
+        }
+        before += tiles;
+    }
+    if (!found) return;  // beyond the last real tile: that part of the padded space is never read
+    const int row_base = start + (rt - before) * QC_TILE;
+    const int64_t k0 = (int64_t)blockIdx.x * QC_TILE;
+    const int64_t col = k0 + (t & 15) * 8;
+    const bool col_ok = col < a.C;
+    float v[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int pos = row_base + (t >> 4) * 8 + i;
+        if (col_ok && pos < end) {
+            const int64_t src = a.index ? a.index[pos] : pos;
+            if (SRC == SRC_PLAIN) {
+                Elem<DT>::load8((const T *)a.x + src * a.ldx + col, v[i]);
+                if (a.row_scale) {
+                    const int si = a.scale_index ? a.scale_index[pos] : pos;
+                    const float sc = a.scale_f32 ? ((const float *)a.row_scale)[si] : Elem<DT>::load1((const T *)a.row_scale + si);
+#pragma unroll
+                    for (int c = 0; c < 8; c++) v[i][c] *= sc;
+                }
+            } else {
+                float g[8], u[8];
+                Elem<DT>::load8((const T *)a.x + src * a.ldx + col, g);
+                Elem<DT>::load8((const T *)a.x + src * a.ldx + a.C + col, u);
+#pragma unroll
+                for (int c = 0; c < 8; c++) v[i][c] = g[c] * sigmoid_fast(g[c]) * u[c];
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
+        }
+    }
+    quant_tile<false>(v, o, mpad, a.C, (int64_t)rt * QC_TILE, k0, tile, tscale);
+}
+
 }  // namespace mx
 
 // ------------------------------------------------------------------------------------
@@ -580,6 +659,36 @@ extern "C" int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const v
     if (H % 128) o.pack_row_scales = 0;  // the up half's scale columns start at H/32: keep dword stores aligned
     if (dtype == MX_BF16) swiglu_bwd_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);
     else swiglu_bwd_quant_dual_kernel<MX_FP16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+extern "C" int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, int64_t C, int source,
+                                        const int32_t *index, const void *row_scale, int row_scale_dtype,
+                                        const int32_t *scale_index, const int32_t *offsets, int64_t E, int64_t M,
+                                        uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream) {
+    if (M < 0 || C < 0 || E <= 0 || E >= (1 << 20) || M >= 0x7FFFFFFF || C >= 0x7FFFFFFF) return MX_EINVAL;
+    if (source != SRC_PLAIN && source != SRC_SWIGLU) return MX_EINVAL;
+    const int64_t tiles = (M + QC_TILE - 1) / QC_TILE + E;
+    const int64_t mpad = tiles * QC_TILE;
+    if (ldqT < mpad || ldsT < mpad / MX_BLOCK || ldx < (source == SRC_SWIGLU ? 2 * C : C)) return MX_EINVAL;
+    if (row_scale && row_scale_dtype != MX_FP32 && row_scale_dtype != dtype) return MX_EINVAL;
+    if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
+    if (C % 8 || !aligned(x, 16) || (ldx * 2) % 16 || !aligned(qT, 16) || ldqT % 16 || tiles > 65535) return MX_EUNSUPPORTED;
+    if (C == 0) return MX_OK;
+    GroupedQuantArgs a;
+    a.x = x, a.ldx = ldx, a.C = (int)C, a.index = index, a.row_scale = row_scale, a.scale_index = scale_index;
+    a.scale_f32 = row_scale_dtype == MX_FP32, a.offsets = offsets, a.E = (int)E;
+    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, nullptr, 0, nullptr, 0);
+    dim3 grid((unsigned)((C + QC_TILE - 1) / QC_TILE), (unsigned)tiles);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MX_BF16) {
+        if (source == SRC_PLAIN) quant_cols_grouped_kernel<MX_BF16, SRC_PLAIN><<<grid, dim3(256), 0, st>>>(a, o, mpad);
+        else quant_cols_grouped_kernel<MX_BF16, SRC_SWIGLU><<<grid, dim3(256), 0, st>>>(a, o, mpad);
+    } else {
+        if (source == SRC_PLAIN) quant_cols_grouped_kernel<MX_FP16, SRC_PLAIN><<<grid, dim3(256), 0, st>>>(a, o, mpad);
+        else quant_cols_grouped_kernel<MX_FP16, SRC_SWIGLU><<<grid, dim3(256), 0, st>>>(a, o, mpad);
+    }
     MX_LAUNCH_CHECK();
     return MX_OK;
 }

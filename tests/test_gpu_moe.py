@@ -1,0 +1,347 @@
+"""Routed experts in MXFP8 against the CPU oracle: grouped GEMM, the fused expert kernels, WGRAD.
+
+Oracle = per-expert loop over the offset table of dequantize-then-matmul in fp64 on operands
+quantized by the oracle; 1e-2 relative Frobenius for 16-bit outputs.  Outputs accumulated with
+atomics (out, dx, dgate) are compared by norm, never bitwise: their summation order is free.
+"""
+
+import pytest
+import torch
+
+from conftest import SEED
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = 1e-2
+F8 = torch.float8_e4m3fn
+
+
+def _dev(q, s):
+    return q.to(DEV).view(F8), s.to(DEV)
+
+
+def _routing(counts, top_k, tokens, seed=SEED):
+    """offsets/order/token_of for given per-expert counts: position m of expert e takes distinct tokens."""
+    g = torch.Generator().manual_seed(seed)
+    offsets = torch.zeros(len(counts) + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    m = int(offsets[-1])
+    token_of = torch.empty(m, dtype=torch.int32)
+    slot = torch.zeros(tokens, dtype=torch.int64)  # how many experts each token already has
+    order = torch.empty(m, dtype=torch.int32)
+    for e, c in enumerate(counts):
+        free = (slot < top_k).nonzero().flatten()
+        pick = free[torch.randperm(free.numel(), generator=g)[:c]]
+        assert pick.numel() == c
+        lo = int(offsets[e])
+        token_of[lo : lo + c] = pick.int()
+        order[lo : lo + c] = (pick * top_k + slot[pick]).int()
+        slot[pick] += 1
+    return offsets, order, token_of
+
+
+COUNT_CASES = [
+    [300, 0, 1, 257, 0, 130],  # empty, single-row, just over a tile
+    [64, 64, 64, 64],
+    [0, 0, 5, 0],
+    [700],
+]
+
+
+@pytest.mark.parametrize("counts", COUNT_CASES)
+@pytest.mark.parametrize("use_index", [False, True])
+def test_grouped_gemm(oracle, counts, use_index):
+    from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_gemm, grouped_mxfp8_reference
+
+    g = torch.Generator().manual_seed(SEED)
+    e, n, k = len(counts), 320, 256
+    m = sum(counts)
+    tokens = max(m, 8) if not use_index else 200
+    x = torch.randn(tokens, k, generator=g).bfloat16()
+    w = (torch.randn(e, n, k, generator=g) * 0.05).bfloat16()
+    xq, xs = oracle.quantize_rows(x)
+    wq, ws = oracle.quantize_rows(w.reshape(e * n, k))
+    wq, ws = wq.view(e, n, k), ws.view(e, n, k // 32)
+    offsets = torch.zeros(e + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    index = torch.randint(0, tokens, (m,), generator=g).int() if use_index else None
+    ref = oracle.grouped_gemm_nt(xq, xs, wq, ws, offsets, index)
+    got = grouped_mxfp8_gemm(*_dev(xq, xs), *_dev(wq, ws), offsets.to(DEV), None if index is None else index.to(DEV),
+                             rows=m)
+    assert got.shape == (m, n) and got.dtype == torch.bfloat16
+    assert oracle.rel_error(got.cpu(), ref) < TOL
+    # the reference's own precision oracle, run on the device tensors, agrees with ours
+    ref2 = grouped_mxfp8_reference(*_dev(xq, xs), *_dev(wq, ws), offsets.to(DEV), None if index is None else index.to(DEV))
+    assert oracle.rel_error(ref2.cpu(), ref) < 1e-12
+    # fp32 output: nothing but the MFMA's internal adder between us and fp64
+    got32 = grouped_mxfp8_gemm(*_dev(xq, xs), *_dev(wq, ws), offsets.to(DEV), None if index is None else index.to(DEV),
+                               out_dtype=torch.float32, rows=m)
+    assert oracle.rel_error(got32.cpu(), ref) < 1e-4
+
+
+def test_grouped_gemm_sentinel_rows_untouched_and_errors(oracle):
+    from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_gemm
+
+    g = torch.Generator().manual_seed(SEED)
+    e, n, k, m = 3, 128, 128, 100
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(e, n, k, generator=g) * 0.05).bfloat16()
+    xq, xs = oracle.quantize_rows(x)
+    wq, ws = oracle.quantize_rows(w.reshape(e * n, k))
+    wq, ws = wq.view(e, n, k), ws.view(e, n, k // 32)
+    offsets = torch.tensor([0, 30, 30, 70], dtype=torch.int32)  # rows 70..99 belong to no real expert
+    out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=DEV)
+    grouped_mxfp8_gemm(*_dev(xq, xs), *_dev(wq, ws), offsets.to(DEV), out=out)
+    ref = oracle.grouped_gemm_nt(xq, xs, wq, ws, offsets)
+    assert oracle.rel_error(out[:70].cpu(), ref) < TOL
+    assert (out[70:] == 7.0).all()
+    # K not a multiple of 128: the generic kernel
+    xq2, xs2, wq2, ws2 = xq[:, :96].contiguous(), xs[:, :3].contiguous(), wq[:, :, :96].contiguous(), ws[:, :, :3].contiguous()
+    got = grouped_mxfp8_gemm(*_dev(xq2, xs2), *_dev(wq2, ws2), offsets.to(DEV), rows=70)
+    assert oracle.rel_error(got.cpu(), oracle.grouped_gemm_nt(xq2, xs2, wq2, ws2, offsets)) < TOL
+    with pytest.raises(ValueError):
+        grouped_mxfp8_gemm(*_dev(xq[:, :64], xs[:, :2]), *_dev(wq, ws), offsets.to(DEV))
+    with pytest.raises(ValueError):
+        grouped_mxfp8_gemm(*_dev(xq, xs), *_dev(wq, ws[:, :, :2]), offsets.to(DEV))
+    with pytest.raises(ValueError):
+        grouped_mxfp8_gemm(*_dev(xq, xs), *_dev(wq, ws), offsets.to(DEV), out=torch.empty(3, 3, device=DEV))
+
+
+def _padded_cols_ref(oracle, rows_fp32, offsets, dtype=torch.bfloat16):
+    """Oracle for the grouped token-axis quantizer: each expert's rows padded to a multiple of 128, then quantize_cols."""
+    off = offsets.tolist()
+    e = len(off) - 1
+    mpad = (-(-rows_fp32.shape[0] // 128) + e) * 128
+    c = rows_fp32.shape[1]
+    q = torch.zeros(c, mpad, dtype=torch.uint8)
+    s = torch.zeros(c, mpad // 32, dtype=torch.uint8)
+    valid = torch.zeros(mpad, dtype=torch.bool)
+    pos = 0
+    for i in range(e):
+        cnt = off[i + 1] - off[i]
+        tiles = -(-cnt // 128)
+        if tiles == 0:
+            continue
+        block = torch.zeros(tiles * 128, c)
+        block[:cnt] = rows_fp32[off[i] : off[i + 1]]
+        bq, bs = oracle.quantize_cols(block)
+        q[:, pos : pos + tiles * 128] = bq
+        s[:, pos // 32 : (pos + tiles * 128) // 32] = bs
+        valid[pos : pos + tiles * 128] = True
+        pos += tiles * 128
+    return q, s, valid
+
+
+@pytest.mark.parametrize("counts", COUNT_CASES[:3])
+def test_grouped_token_axis_quantizer_and_wgrad(oracle, counts):
+    from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_wgrad, quantize_mx_cols_grouped
+
+    g = torch.Generator().manual_seed(SEED)
+    e, m = len(counts), sum(counts)
+    tokens, n, k = 400, 256, 192
+    offsets = torch.zeros(e + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    a = (torch.randn(m, n, generator=g) * 1e-2).bfloat16()
+    x = torch.randn(tokens, k, generator=g).bfloat16()
+    index = torch.randint(0, tokens, (m,), generator=g).int()
+    scale = (torch.rand(m * 2, generator=g) + 0.5).bfloat16()
+    sidx = torch.randperm(m * 2, generator=g)[:m].int()
+    # plain
+    atq, ats = quantize_mx_cols_grouped(a.to(DEV), offsets.to(DEV), m)
+    rq, rs, valid = _padded_cols_ref(oracle, a.float(), offsets)
+    vs = valid.view(-1, 32)[:, 0]
+    assert torch.equal(atq.view(torch.uint8).cpu()[:, valid], rq[:, valid])
+    assert torch.equal(ats.cpu()[:, vs], rs[:, vs])
+    # gathered rows times a gathered row scale (fp32 product, then quantized)
+    btq, bts = quantize_mx_cols_grouped(x.to(DEV), offsets.to(DEV), m, index=index.to(DEV), row_scale=scale.to(DEV),
+                                        scale_index=sidx.to(DEV))
+    rows = x[index.long()].float() * scale[sidx.long()].float()[:, None]
+    bq_ref, bs_ref, _ = _padded_cols_ref(oracle, rows, offsets)
+    assert torch.equal(btq.view(torch.uint8).cpu()[:, valid], bq_ref[:, valid])
+    assert torch.equal(bts.cpu()[:, vs], bs_ref[:, vs])
+    # swiglu source
+    pre = torch.randn(m, 2 * 128, generator=g).bfloat16()
+    htq, hts = quantize_mx_cols_grouped(pre.to(DEV), offsets.to(DEV), m, swiglu=True)
+    gg, vv = pre.float().chunk(2, dim=-1)
+    hq_ref, hs_ref, _ = _padded_cols_ref(oracle, gg * torch.sigmoid(gg) * vv, offsets)
+    assert (htq.view(torch.uint8).cpu()[:, valid] != hq_ref[:, valid]).float().mean() < 5e-3
+    # WGRAD on the token-axis operands: per-expert A^T B of the dequantized padded blocks
+    dw = grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets.to(DEV), m)
+    assert dw.shape == (e, n, k)
+    ad = oracle.dequant(rq.T.contiguous().T, rs)  # (n, mpad)
+    bd = oracle.dequant(bq_ref, bs_ref)  # (k, mpad)
+    pos = 0
+    for i, cnt in enumerate(counts):
+        tiles = -(-cnt // 128)
+        ref = ad[:, pos : pos + tiles * 128] @ bd[:, pos : pos + tiles * 128].T
+        pos += tiles * 128
+        if cnt == 0:
+            assert (dw[i] == 0).all()
+        else:
+            assert oracle.rel_error(dw[i].cpu(), ref) < TOL, (i, cnt)
+
+
+def _expert_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
+    """The fused path's arithmetic restated with oracle primitives, stage by stage."""
+    e, two_h, dim = w_in.shape
+    hid = two_h // 2
+    off = offsets.tolist()
+    m = off[-1]
+    t_idx, p_idx = token_of.long()[:m], order.long()[:m]
+
+    def stacked(w):
+        q, s = ora.quantize_rows(w.reshape(-1, w.shape[-1]))
+        return q.view(*w.shape), s.view(*w.shape[:-1], w.shape[-1] // 32)
+
+    in_f, out_f = stacked(w_in), stacked(w_out)
+    in_d, out_d = stacked(w_in.transpose(1, 2).contiguous()), stacked(w_out.transpose(1, 2).contiguous())
+    xq, xs = ora.quantize_rows(x)
+    pre = ora.grouped_gemm_nt(xq, xs, *in_f, offsets, t_idx).bfloat16()
+    g, v = pre.float().chunk(2, dim=-1)
+    h = g * torch.sigmoid(g) * v
+    hq, hs = ora.quantize_rows(h)
+    y = ora.grouped_gemm_nt(hq, hs, *out_f, offsets)
+    gate_m = gate.float()[p_idx].double()
+    out = torch.zeros(x.shape[0], dim, dtype=torch.float64).index_add_(0, t_idx, y * gate_m[:, None])
+    # backward
+    dq, ds = ora.quantize_rows(dout)
+    acc = ora.grouped_gemm_nt(dq, ds, *out_d, offsets, t_idx)  # (m, hid)
+    dgate = torch.zeros(gate.numel(), dtype=torch.float64).index_add_(0, p_idx, (acc * ora.dequant(hq, hs)).sum(-1))
+    dh = (acc * gate_m[:, None]).float()
+    sg = torch.sigmoid(g)
+    dpre = torch.cat([dh * v * sg * (1 + g * (1 - sg)), dh * g * sg], dim=-1)
+    pq, ps = ora.quantize_rows(dpre)
+    dx = torch.zeros(x.shape[0], dim, dtype=torch.float64).index_add_(0, t_idx, ora.grouped_gemm_nt(pq, ps, *in_d, offsets))
+    # WGRAD on token-axis blocks inside each expert's segment
+    a_out = dout.float()[t_idx] * gate.float()[p_idx][:, None]
+    dw_out = torch.zeros(e, dim, hid, dtype=torch.float64)
+    dw_in = torch.zeros(e, two_h, dim, dtype=torch.float64)
+    dpre16 = dpre.bfloat16().float()
+    xg = x.float()[t_idx]
+    for i in range(e):
+        lo, hi = off[i], off[i + 1]
+        if hi == lo:
+            continue
+        pad = -(hi - lo) % 32
+
+        def qc(rows):
+            rows = torch.nn.functional.pad(rows, (0, 0, 0, pad))
+            return ora.quantize_cols(rows)
+
+        dw_out[i] = ora.gemm_nt(*qc(a_out[lo:hi]), *qc(h[lo:hi]))
+        dw_in[i] = ora.gemm_nt(*qc(dpre16[lo:hi]), *qc(xg[lo:hi]))
+    return dict(out=out, pre=pre, hq=hq, hs=hs, dx=dx, dgate=dgate, dw_in=dw_in, dw_out=dw_out)
+
+
+@pytest.mark.parametrize("counts,top_k", [([300, 0, 1, 257, 0, 130], 2), ([256, 256], 1)])
+@pytest.mark.parametrize("dout_scale", [1.0, 2.0**-20])
+def test_fused_experts_fwd_bwd(oracle, counts, top_k, dout_scale):
+    from kohakuwullm_amd.kernels.mxfp8.moe import (
+        MXFP8ExpertWeights,
+        mxfp8_moe_experts,
+        mxfp8_moe_experts_reference,
+        mxfp8_moe_experts_unfused,
+    )
+
+    g = torch.Generator().manual_seed(SEED)
+    e, tokens, dim, hid = len(counts), 512, 256, 128
+    offsets, order, token_of = _routing(counts, top_k, tokens)
+    x = torch.randn(tokens, dim, generator=g).bfloat16()
+    w_in = (torch.randn(e, 2 * hid, dim, generator=g) * 0.06).bfloat16()
+    w_out = (torch.randn(e, dim, hid, generator=g) * 0.06).bfloat16()
+    gate = (torch.rand(tokens * top_k, generator=g) * 0.5 + 0.5).bfloat16()
+    dout = (torch.randn(tokens, dim, generator=g) * dout_scale).bfloat16()
+    ref = _expert_oracle(oracle, x, w_in, w_out, gate, token_of, order, offsets, dout)
+
+    def run(fn):
+        xd, wi, wo, gd = (t.to(DEV).requires_grad_(True) for t in (x, w_in, w_out, gate))
+        packed = MXFP8ExpertWeights(wi.detach(), wo.detach())
+        out = fn(xd, wi, wo, gd, token_of.to(DEV), order.to(DEV), offsets.to(DEV), packed)
+        assert out.grad_fn is not None and out.shape == (tokens, dim) and out.dtype == torch.bfloat16
+        out.backward(dout.to(DEV))
+        return out.detach().cpu(), xd.grad.cpu(), wi.grad.cpu(), wo.grad.cpu(), gd.grad.cpu()
+
+    out, dx, dw_in, dw_out, dgate = run(mxfp8_moe_experts)
+    assert oracle.rel_error(out, ref["out"]) < TOL
+    assert oracle.rel_error(dx, ref["dx"]) < TOL
+    assert oracle.rel_error(dgate, ref["dgate"]) < TOL
+    assert oracle.rel_error(dw_out, ref["dw_out"]) < TOL
+    assert oracle.rel_error(dw_in, ref["dw_in"]) < TOL
+    for i, c in enumerate(counts):
+        if c == 0:
+            assert (dw_in[i] == 0).all() and (dw_out[i] == 0).all()
+    assert dgate.dtype == gate.dtype and dw_in.dtype == torch.bfloat16
+
+    # structural reference without quantization (autograd in fp32): the gap is the e4m3 error of the chain
+    xf, wif, wof, gf = (t.float().requires_grad_(True) for t in (x, w_in, w_out, gate))
+    yf = mxfp8_moe_experts_reference(xf, wif, wof, gf, token_of, order, offsets)
+    yf.backward(dout.float())
+    assert oracle.rel_error(out, yf) < 0.08
+    assert oracle.rel_error(dx, xf.grad) < 0.12
+    assert oracle.rel_error(dw_in, wif.grad) < 0.12
+    assert oracle.rel_error(dw_out, wof.grad) < 0.12
+    assert oracle.rel_error(dgate, gf.grad) < 0.12
+
+    # the unfused twin computes the same function through differently placed casts (16-bit h and
+    # dh round trips, the gate applied before the dgrad quantizer): its forward sits within the
+    # 16-bit round trip of the fused oracle, its gradients within the e4m3 error of the exact ones
+    out_u, dx_u, dw_in_u, dw_out_u, dgate_u = run(mxfp8_moe_experts_unfused)
+    assert oracle.rel_error(out_u, ref["out"]) < 2e-2
+    assert oracle.rel_error(dx_u, xf.grad) < 0.12
+    assert oracle.rel_error(dw_in_u, wif.grad) < 0.12
+    assert oracle.rel_error(dw_out_u, wof.grad) < 0.12
+    assert oracle.rel_error(dgate_u, gf.grad) < 0.12
+
+
+def test_gemm1_intermediates(oracle):
+    """GEMM1's three outputs against the oracle: pre is the rounded accumulator, h is quantized from fp32."""
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, launch_gemm1
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator().manual_seed(SEED)
+    counts, top_k = [200, 0, 56], 1
+    e, tokens, dim, hid = len(counts), 256, 128, 160
+    offsets, order, token_of = _routing(counts, top_k, tokens)
+    x = torch.randn(tokens, dim, generator=g).bfloat16()
+    w_in = (torch.randn(e, 2 * hid, dim, generator=g) * 0.08).bfloat16()
+    w_out = (torch.randn(e, dim, hid, generator=g) * 0.08).bfloat16()
+    gate = torch.ones(tokens, dtype=torch.bfloat16)
+    ref = _expert_oracle(oracle, x, w_in, w_out, gate, token_of, order, offsets, torch.zeros(tokens, dim).bfloat16())
+    packed = MXFP8ExpertWeights(w_in.to(DEV), w_out.to(DEV))
+    m = sum(counts)
+    xq, xs = quantize_mx(x.to(DEV))
+    hq = torch.zeros(m, hid, device=DEV, dtype=F8)
+    hs = torch.zeros(m, hid // 32, device=DEV, dtype=torch.uint8)
+    pre = torch.zeros(m, 2 * hid, device=DEV, dtype=torch.bfloat16)
+    launch_gemm1(xq, xs, token_of.to(DEV), *packed.in_fwd, hq, hs, pre, offsets.to(DEV), hid, dim, torch.bfloat16)
+    assert oracle.rel_error(pre.cpu(), ref["pre"].double()) < 2e-3  # same bf16 values up to accumulation-order ulps
+    hd = oracle.dequant(hq.view(torch.uint8).cpu(), hs.cpu())
+    assert oracle.rel_error(hd, oracle.dequant(ref["hq"], ref["hs"])) < 2e-2
+    assert (hs.cpu() != ref["hs"]).float().mean() < 0.02
+
+
+def test_expert_call_contract():
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, mxfp8_moe_experts
+
+    e, tokens, dim, hid = 2, 64, 128, 128
+    x = torch.randn(tokens, dim, device=DEV, dtype=torch.bfloat16)
+    w_in = torch.randn(e, 2 * hid, dim, device=DEV, dtype=torch.bfloat16)
+    w_out = torch.randn(e, dim, hid, device=DEV, dtype=torch.bfloat16)
+    packed = MXFP8ExpertWeights(w_in, w_out)
+    assert packed.in_fwd[0].shape == (e, 2 * hid, dim) and packed.in_dgrad[0].shape == (e, dim, 2 * hid)
+    assert packed.out_fwd[0].shape == (e, dim, hid) and packed.out_dgrad[0].shape == (e, hid, dim)
+    assert packed.in_fwd[0].dtype == F8 and packed.in_fwd[1].dtype == torch.uint8
+    tok = torch.arange(tokens, device=DEV, dtype=torch.int32)
+    off = torch.tensor([0, 32, 64], device=DEV, dtype=torch.int32)
+    gate = torch.ones(tokens, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        mxfp8_moe_experts(x.float(), w_in, w_out, gate, tok, tok, off, packed)
+    with pytest.raises(ValueError):
+        mxfp8_moe_experts(x.t().contiguous().t(), w_in[:, :, :64], w_out, gate, tok, tok, off, packed)
+    with pytest.raises(ValueError):
+        mxfp8_moe_experts(torch.randn(dim, tokens, device=DEV, dtype=torch.bfloat16).t(), w_in, w_out, gate, tok, tok, off, packed)
+    with pytest.raises(ValueError):
+        mxfp8_moe_experts(x, w_in, w_out, gate, tok, tok[:10], off, packed)
+    y = mxfp8_moe_experts(x, w_in, w_out, gate, tok, tok, off, packed)  # no grad needed: inference path
+    assert y.grad_fn is None and y.shape == (tokens, dim)
