@@ -1,0 +1,66 @@
+"""The C ABI: every function include/mxfp8_hip.h declares is exported, typed in the binding, and arity-checked.
+
+No kernel runs here (no GPU needed); the library only has to load.
+"""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mxfp8_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = {}
+    for m in re.finditer(r"\b(?:int|const char \*)\s*(mx_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        params = m.group(2).strip()
+        decls[m.group(1)] = 0 if params in ("", "void") else params.count(",") + 1
+    return decls
+
+
+def test_header_parses_to_the_expected_surface():
+    names = set(_declared())
+    assert {"mx_quantize_rows", "mx_quantize_cols", "mx_quantize_dual", "mx_gemm_nt", "mx_grouped_gemm_nt",
+            "mx_experts_gemm1", "mx_experts_scatter_gemm", "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt",
+            "mx_quantize_cols_grouped", "mx_swiglu_quantize_rows", "mx_swiglu_quantize_dual",
+            "mx_swiglu_bwd_quantize_dual", "mx_abi_version", "mx_strerror", "mx_device_supported"} <= names
+
+
+def test_library_exports_every_declared_symbol():
+    from kohakuwullm_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} is not built: run __graft_entry__.build()")
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+
+
+def test_binding_matches_header():
+    from kohakuwullm_amd import _lib
+
+    declared = _declared()
+    assert set(_lib.SIGNATURES) == set(declared)
+    for name, (restype, argtypes) in _lib.SIGNATURES.items():
+        assert len(argtypes) == declared[name], f"{name}: binding has {len(argtypes)} args, header {declared[name]}"
+    lib = _lib.load()
+    assert lib.mx_abi_version() == 1
+    assert b"invalid" in lib.mx_strerror(-1) and lib.mx_strerror(0) == b"ok"
+
+
+def test_entry_points_validate_before_launch():
+    """Contract violations are refused with MX_EINVAL before any kernel is launched (null pointers are never touched)."""
+    from kohakuwullm_amd import _lib
+
+    lib = _lib.load()
+    assert lib.mx_quantize_rows(None, 0, 4, 48, 48, 1, None, 48, None, 1, None) == _lib.MX_EINVAL  # K % 32
+    assert lib.mx_quantize_cols(None, 0, 48, 64, 64, None, 48, None, 1, None) == _lib.MX_EINVAL  # M % 32
+    assert lib.mx_quantize_rows(None, 0, 0, 64, 64, 1, None, 64, None, 2, None) == _lib.MX_OK  # empty
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 48, 48, 1, 48, 1, 4, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 32, 2, 64, 2, 4, 0, None) == _lib.MX_EINVAL  # lda < K
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 64, 64, 2, 64, 2, 4, 0, None) == _lib.MX_OK
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 64, 2, 64, 2, 4, 1, None) == _lib.MX_EINVAL  # accumulate needs fp32

@@ -345,3 +345,42 @@ def test_expert_call_contract():
         mxfp8_moe_experts(x, w_in, w_out, gate, tok, tok[:10], off, packed)
     y = mxfp8_moe_experts(x, w_in, w_out, gate, tok, tok, off, packed)  # no grad needed: inference path
     assert y.grad_fn is None and y.shape == (tokens, dim)
+
+
+def test_moe_module_swap_and_train_step(oracle):
+    """MoEMLP through swap_mxfp8: declaration protocol, fused vs eager outputs, refresh contract."""
+    from kohakuwullm_amd.models.moe import MoEMLP, expert_sort
+    from kohakuwullm_amd.models.mxfp8_swap import refresh_mxfp8_weights, swap_mxfp8
+    from kohakuwullm_amd.registry import MOE, build
+
+    torch.manual_seed(0)
+    moe = build("moe", MOE, dim=256, hidden=128, num_experts=8, top_k=2).to(DEV)
+    x = torch.randn(4, 96, 256, device=DEV, dtype=torch.bfloat16)
+    y_eager = moe(x)
+    report = swap_mxfp8(moe)
+    assert not report.blocking, report.summary()
+    assert sorted(report.swapped) == ["w_in", "w_out"] and report.by_design == ["router.weight"]
+    assert report.mac["fp8"] == 2 * (2 * 128 * 256 + 256 * 128)
+    assert refresh_mxfp8_weights(moe) == 1
+    assert list(moe.state_dict()) == ["w_in", "w_out", "router.weight"]
+    xg = x.clone().requires_grad_(True)
+    y = moe(xg)
+    assert y.shape == x.shape and oracle.rel_error(y.float().cpu(), y_eager.float().cpu()) < 0.08
+    y.float().square().mean().backward()
+    for name in ("w_in", "w_out"):
+        grad = getattr(moe, name).grad
+        assert grad is not None and grad.abs().sum() > 0
+    assert moe.router.weight.grad is not None and xg.grad.abs().sum() > 0
+    moe.float()
+    assert moe._packed is None
+    # the unfused path is selected before conversion
+    moe2 = MoEMLP(256, 128, 8, 2, mxfp8_expert_path="unfused").to(DEV)
+    swap_mxfp8(moe2)
+    assert moe2._routed == moe2._routed_mxfp8_unfused and moe2(x).shape == x.shape
+    bad = MoEMLP(256, 48, 4, 2).to(DEV)
+    assert swap_mxfp8(bad).blocking
+    # dispatch format: stable order inside an expert, offsets = cumsum(counts)
+    idx = torch.tensor([2, 0, 2, 1, 0, 2], device=DEV)
+    counts = torch.tensor([2, 1, 3], device=DEV, dtype=torch.int32)
+    offsets, order, token_of, _ = expert_sort(idx, counts, 2, 3)
+    assert offsets.tolist() == [0, 2, 3, 6] and order.tolist() == [1, 4, 3, 0, 2, 5] and token_of.tolist() == [0, 2, 1, 0, 1, 2]
