@@ -51,6 +51,93 @@ def make_inputs(tokens: int):
     return x, torch.cat([w_gate, w_up], 0), w_down, dy
 
 
+def make_attention_inputs(tokens: int = 32768, dim: int = 2048, heads: int = 16, kv_heads: int = 4, head_dim: int = 128):
+    """BASELINE configs[2]: GQA attention projections.  Hidden N(0,1); W_qkv [(heads+2*kv)*hd, dim], W_o [dim, dim] N(0,0.02)."""
+    import torch
+
+    g = torch.Generator().manual_seed(SEED)
+    hid = torch.randn(tokens, dim, generator=g).bfloat16()
+    w_qkv = (torch.randn((heads + 2 * kv_heads) * head_dim, dim, generator=g) * 0.02).bfloat16()
+    w_o = (torch.randn(dim, heads * head_dim, generator=g) * 0.02).bfloat16()
+    d_qkv = (torch.randn(tokens, w_qkv.shape[0], generator=g) * 1e-2).bfloat16()
+    d_o = (torch.randn(tokens, dim, generator=g) * 1e-2).bfloat16()
+    return hid, w_qkv, w_o, d_qkv, d_o
+
+
+def zipf_counts(num_experts: int = 64, total: int = 98304, cap: int = 16384, s: float = 1.1):
+    """Per-expert row counts ~ Zipf(s), summing to `total`, each <= cap, at least one expert empty."""
+    import numpy as np
+
+    z = np.random.Generator(np.random.PCG64(SEED)).zipf(s, num_experts).astype(np.float64)
+    c = np.floor(total * z / z.sum()).astype(np.int64)
+    c = np.minimum(c, cap)
+    order = np.argsort(-c, kind="stable")
+    rem = total - int(c.sum())
+    i = 0
+    while rem > 0:  # push the remainder / overflow to the next-largest experts
+        e = order[i % num_experts]
+        add = min(cap - int(c[e]), rem)
+        c[e] += add
+        rem -= add
+        i += 1
+    if (c == 0).sum() == 0:
+        small, big = int(np.argmin(c)), int(np.argmax(np.where(c < cap, c, -1)))
+        c[big] += c[small]
+        c[small] = 0
+    assert int(c.sum()) == total and (c <= cap).all() and (c == 0).any()
+    return [int(v) for v in c]
+
+
+def make_moe_inputs(tokens: int = 16384, dim: int = 1024, hidden: int = 512, num_experts: int = 64, top_k: int = 6):
+    """BASELINE configs[3]: routed experts with Zipf(1.1) loads; sorted position m -> token m mod T, slot m div T."""
+    import torch
+
+    g = torch.Generator().manual_seed(SEED)
+    x = torch.randn(tokens, dim, generator=g).bfloat16()
+    w_in = (torch.randn(num_experts, 2 * hidden, dim, generator=g) * 0.02).bfloat16()
+    w_out = (torch.randn(num_experts, dim, hidden, generator=g) * 0.02).bfloat16()
+    gate = (torch.rand(tokens * top_k, generator=g) * 0.5 + 0.5).bfloat16()
+    dout = (torch.randn(tokens, dim, generator=g) * 1e-2).bfloat16()
+    counts = zipf_counts(num_experts, tokens * top_k, tokens)
+    offsets = torch.zeros(num_experts + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    m = torch.arange(tokens * top_k)
+    token_of = (m % tokens).int()
+    order = (token_of.long() * top_k + m // tokens).int()
+    return x, w_in, w_out, gate, dout, offsets, order, token_of, counts
+
+
+def make_outlier_inputs(n: int = 8192):
+    """BASELINE configs[4]: Student-t(3) activations with 0.1% of channels x200 and injected special blocks."""
+    import torch
+
+    g = torch.Generator().manual_seed(SEED)
+    z = torch.randn(n, n, generator=g)
+    chi = (torch.randn(n, n, 3, generator=g) ** 2).sum(-1) / 3
+    x = z / chi.sqrt()
+    cols = torch.randperm(n, generator=g)[: max(1, n // 1000)]
+    x[:, cols] *= 200.0
+    x = x.bfloat16()
+    blocks = x.view(n, n // 32, 32)
+    nb = n * (n // 32)
+    pick = torch.randperm(nb, generator=g)
+    zero, tiny, big, tie = pick[: nb // 1000], pick[nb // 1000 : nb // 1000 + 64], pick[-128:-64], pick[-64:]
+    flat = blocks.view(nb, 32)
+    flat[zero] = 0.0
+    flat[tiny] = 1e-35
+    flat[big, 0] = 3.0e38
+    flat[big, 1] = -3.0e38
+    j = torch.randint(-20, 20, (64,), generator=g).float()
+    flat[tie] = flat[tie].clamp(-1, 1)
+    flat[tie, 7] = (448.0 * torch.exp2(j)).bfloat16()
+    flat[tie] = torch.minimum(flat[tie].float().abs(), (448.0 * torch.exp2(j))[:, None]).bfloat16() * torch.sign(flat[tie].float()).bfloat16()
+    flat[tie, 7] = (448.0 * torch.exp2(j)).bfloat16()
+    w = (torch.randn(n, n, generator=g) * 0.02).bfloat16()
+    dy = (torch.randn(n, n, generator=g) * 1e-2).bfloat16()
+    special = dict(zero=zero, tiny=tiny, big=big, tie=tie)
+    return x, w, dy, special
+
+
 def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
     """The oracle's formulas with PyTorch CPU ops on the first `sample_tokens` tokens."""
     import torch
@@ -98,11 +185,105 @@ def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
     }
 
 
+GEMM_ENTRIES = ("mx_gemm_nt", "mx_grouped_gemm_nt", "mx_experts_gemm1", "mx_experts_scatter_gemm",
+                "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt")
+
+
+def build_workload(name: str, dev):
+    """Returns (step(i), gflop per step, description, refresh())."""
+    import torch
+
+    from kohakuwullm_amd.kernels.mxfp8.linear import MXFP8Linear
+    from kohakuwullm_amd.kernels.mxfp8.mlp import mxfp8_swiglu_mlp
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, mxfp8_moe_experts
+    from kohakuwullm_amd.kernels.mxfp8.quantize import mxfp8_matmul_pq, quantize_mx, quantize_mx_cols
+
+    ncopies = 4  # rotating activation copies: a step does not find its inputs in the 256 MB last-level cache
+    if name == "ffn":
+        x_h, w_in_h, w_out_h, dy_h = make_inputs(TOKENS)
+        xs = [x_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
+        dys = [dy_h.to(dev) for _ in range(ncopies)]
+        w_in = w_in_h.to(dev).requires_grad_(True)
+        w_out = w_out_h.to(dev).requires_grad_(True)
+        state = {}
+
+        def refresh():
+            state["packed"] = (quantize_mx(w_in.detach()), quantize_mx_cols(w_in.detach()),
+                               quantize_mx(w_out.detach()), quantize_mx_cols(w_out.detach()))
+
+        def step(i):
+            x = xs[i % ncopies]
+            mxfp8_swiglu_mlp(x, w_in, w_out, state["packed"]).backward(dys[i % ncopies])
+            x.grad = w_in.grad = w_out.grad = None
+
+        desc = "dense 546M-class SwiGLU FFN fwd+bwd: tokens 16384, dim 1536, ffn 4096 (BASELINE configs[1])"
+        return step, step_flops(TOKENS) / 1e9, desc, refresh
+    if name == "attn":
+        hid_h, w_qkv_h, w_o_h, d_qkv_h, d_o_h = make_attention_inputs()
+        qkv = MXFP8Linear(w_qkv_h.shape[1], w_qkv_h.shape[0]).to(dev)
+        proj = MXFP8Linear(w_o_h.shape[1], w_o_h.shape[0]).to(dev)
+        with torch.no_grad():
+            qkv.weight.copy_(w_qkv_h.to(dev))
+            proj.weight.copy_(w_o_h.to(dev))
+        xs = [hid_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
+        d_qkv, d_o = d_qkv_h.to(dev), d_o_h.to(dev)
+
+        def refresh():
+            qkv.refresh_quantized_weight()
+            proj.refresh_quantized_weight()
+
+        def step(i):
+            x = xs[i % ncopies]
+            qkv(x).backward(d_qkv)
+            proj(x).backward(d_o)  # the attention core is not run: o_proj sees an activation of the same shape
+            x.grad = qkv.weight.grad = proj.weight.grad = None
+
+        t, d = hid_h.shape
+        gflop = 3 * (2.0 * t * w_qkv_h.shape[0] * d + 2.0 * t * d * d) / 1e9
+        return step, gflop, "GQA attention projections fwd+dgrad+wgrad: tokens 32768, dim 2048, W_qkv 3072x2048, W_o 2048x2048 (BASELINE configs[2])", refresh
+    if name == "moe":
+        x_h, w_in_h, w_out_h, gate_h, dout_h, offsets, order, token_of, counts = make_moe_inputs()
+        xs = [x_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
+        w_in, w_out = w_in_h.to(dev).requires_grad_(True), w_out_h.to(dev).requires_grad_(True)
+        gate = gate_h.to(dev).requires_grad_(True)
+        dout, offsets, order, token_of = dout_h.to(dev), offsets.to(dev), order.to(dev), token_of.to(dev)
+        state = {}
+
+        def refresh():
+            state["packed"] = MXFP8ExpertWeights(w_in.detach(), w_out.detach())
+
+        def step(i):
+            x = xs[i % ncopies]
+            mxfp8_moe_experts(x, w_in, w_out, gate, token_of, order, offsets, state["packed"]).backward(dout)
+            x.grad = w_in.grad = w_out.grad = gate.grad = None
+
+        m, dim, hid = int(sum(counts)), x_h.shape[1], w_out_h.shape[2]
+        return step, 3 * 6.0 * m * dim * hid / 1e9, "routed experts fwd+bwd: 64 experts (Zipf 1.1 loads, 58 empty), top-6, tokens 16384, dim 1024, hidden 512 (BASELINE configs[3])", refresh
+    if name == "outlier":
+        x_h, w_h, dy_h, _ = make_outlier_inputs()
+        x, w, dy = x_h.to(dev), w_h.to(dev), dy_h.to(dev)
+        state = {}
+
+        def refresh():
+            state["w"] = quantize_mx(w)
+
+        def step(i):
+            xq, xs_ = quantize_mx(x)
+            mxfp8_matmul_pq(xq, xs_, *state["w"])
+            mxfp8_matmul_pq(*quantize_mx_cols(dy), *quantize_mx_cols(x))
+
+        n = x_h.shape[0]
+        return step, 2 * 2.0 * n**3 / 1e9, "outlier-stress 8192^3 GEMM, fwd + wgrad, quantizers included (BASELINE configs[4])", refresh
+    raise SystemExit(f"unknown workload {name!r}")
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier"),
+                    help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -111,39 +292,18 @@ def main() -> None:
     import torch
 
     from kohakuwullm_amd import _lib
-    from kohakuwullm_amd.kernels.mxfp8.mlp import mxfp8_swiglu_mlp
-    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx, quantize_mx_cols
 
     dev = torch.device("cuda:0")
     _lib.check(_lib.load().mx_device_supported(0), "mx_device_supported")
-    x_h, w_in_h, w_out_h, dy_h = make_inputs(TOKENS)
-    # Several copies of the activations so consecutive steps do not find their inputs in the
-    # 256 MB last-level cache.
-    ncopies = 4
-    xs = [x_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
-    dys = [dy_h.to(dev) for _ in range(ncopies)]
-    w_in = w_in_h.to(dev).requires_grad_(True)
-    w_out = w_out_h.to(dev).requires_grad_(True)
+    step, gflop, desc, refresh = build_workload(args.workload, dev)
 
-    def refresh():
-        return (quantize_mx(w_in.detach()), quantize_mx_cols(w_in.detach()),
-                quantize_mx(w_out.detach()), quantize_mx_cols(w_out.detach()))
-
-    packed = refresh()
+    refresh()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(10):
-        packed = refresh()
+    for _ in range(5):
+        refresh()
     torch.cuda.synchronize()
-    weight_refresh_ms = (time.perf_counter() - t0) / 10 * 1e3
-
-    def step(i: int) -> None:
-        x = xs[i % ncopies]
-        y = mxfp8_swiglu_mlp(x, w_in, w_out, packed)
-        y.backward(dys[i % ncopies])
-        x.grad = None
-        w_in.grad = None
-        w_out.grad = None
+    weight_refresh_ms = (time.perf_counter() - t0) / 5 * 1e3
 
     for i in range(args.warmup):
         step(i)
@@ -154,7 +314,7 @@ def main() -> None:
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
-    tflops = step_flops(TOKENS) / (ms_per_step * 1e-3) / 1e12
+    tflops = gflop / ms_per_step
 
     # Instrumented pass: the same steps with events around every kernel launch.
     _lib.TIMER = []
@@ -162,15 +322,15 @@ def main() -> None:
         step(i)
     torch.cuda.synchronize()
     records, _lib.TIMER = _lib.TIMER, None
-    gemm = [(w, a.elapsed_time(b)) for n, w, a, b in records if n == "mx_gemm_nt"]
-    quant = [(w, a.elapsed_time(b)) for n, w, a, b in records if n != "mx_gemm_nt"]
-    gemm_flops, gemm_ms = sum(w for w, _ in gemm), sum(t for _, t in gemm)
-    quant_bytes, quant_ms = sum(w for w, _ in quant), sum(t for _, t in quant)
+    gemm = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n in GEMM_ENTRIES]
+    quant = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n not in GEMM_ENTRIES]
+    gemm_flops, gemm_ms = sum(w for _, w, _ in gemm), sum(t for _, _, t in gemm)
+    quant_bytes, quant_ms = sum(w for _, w, _ in quant), sum(t for _, _, t in quant)
     gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
     quant_gbs = quant_bytes / (quant_ms * 1e-3) / 1e9
 
     out = {
-        "metric": "MXFP8 linear fwd+bwd TFLOP/s (dense SwiGLU FFN, quantizers included)",
+        "metric": "MXFP8 linear fwd+bwd TFLOP/s (quantizers included)",
         "value": round(tflops, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -183,13 +343,13 @@ def main() -> None:
         "dtype": "mxfp8 (e4m3 x e4m3 with ue8m0 per-32 scales, fp32 accumulate, bf16 out)",
         "data": "synthetic",
         "config": {
-            "workload": "dense 546M-class SwiGLU FFN fwd+bwd: tokens 16384, dim 1536, ffn 4096 (BASELINE configs[1])",
-            "gflop_per_step": round(step_flops(TOKENS) / 1e9, 1),
-            "products": "fwd 2, dgrad 2, wgrad 2 (all MXFP8, wgrad on token-axis blocks)",
+            "workload": desc,
+            "gflop_per_step": round(gflop, 1),
+            "products": "fwd, dgrad and wgrad all in MXFP8 (wgrad on token-axis blocks)",
         },
         "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4),
         "roofline": {
-            "kernel": "gemm_nt_kernel (mx_gemm_nt)",
+            "kernel": "block-scaled MFMA GEMM kernels (" + ", ".join(sorted({n for n, _, _ in gemm})) + ")",
             "bound": "mfma",
             "achieved": round(gemm_tflops, 2),
             "peak": MFMA_PEAK_TFLOPS,
@@ -201,7 +361,7 @@ def main() -> None:
             "gflop_per_launch": round(gemm_flops / len(gemm) / 1e9, 2),
         },
         "quantizer": {
-            "kernels": "mx_quantize_dual, mx_swiglu_quantize_dual, mx_swiglu_bwd_quantize_dual",
+            "kernels": ", ".join(sorted({n for n, _, _ in quant})),
             "bound": "hbm",
             "achieved": round(quant_gbs, 1),
             "peak": HBM_PEAK_GBS,
@@ -213,7 +373,7 @@ def main() -> None:
         },
         "weight_refresh_ms": round(weight_refresh_ms, 4),
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload == "ffn":
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 
