@@ -185,7 +185,7 @@ def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
     }
 
 
-GEMM_ENTRIES = ("mx_gemm_nt", "mx_grouped_gemm_nt", "mx_experts_gemm1", "mx_experts_scatter_gemm",
+GEMM_ENTRIES = ("mx_gemm_nt", "mx_gemm_nt_batch", "mx_grouped_gemm_nt", "mx_experts_gemm1", "mx_experts_scatter_gemm",
                 "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt")
 
 
@@ -285,6 +285,7 @@ def main() -> None:
     ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier"),
                     help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this path is built and run on a single GPU (--gpus 1)")
@@ -322,6 +323,14 @@ def main() -> None:
         step(i)
     torch.cuda.synchronize()
     records, _lib.TIMER = _lib.TIMER, None
+    if args.breakdown:
+        per_step = len(records) // args.steps
+        for j in range(per_step):
+            ts = sorted(records[i * per_step + j][2].elapsed_time(records[i * per_step + j][3]) for i in range(args.steps))
+            name, work = records[j][0], records[j][1]
+            rate = work / (ts[len(ts) // 2] * 1e-3)
+            print(f"  {j:2d} {name:28s} median {ts[len(ts) // 2] * 1e3:8.1f} us   "
+                  + (f"{rate / 1e12:7.1f} TFLOP/s" if name in GEMM_ENTRIES else f"{rate / 1e9:7.0f} GB/s"), file=sys.stderr)
     gemm = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n in GEMM_ENTRIES]
     quant = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n not in GEMM_ENTRIES]
     gemm_flops, gemm_ms = sum(w for _, w, _ in gemm), sum(t for _, _, t in gemm)

@@ -2,11 +2,17 @@
  * libmxfp8_hip -- MXFP8 (e4m3 + UE8M0 per-32) linear path for AMD MI355X (gfx950).
  *
  * C ABI.  Every entry point
- *   - takes raw DEVICE pointers, sizes and strides; never allocates, frees or
- *     synchronises; launches on the stream the caller passes (a hipStream_t
- *     travelling as void*; NULL = the default stream);
+ *   - takes raw DEVICE pointers, sizes and strides; never synchronises or frees;
+ *     launches on the stream the caller passes (a hipStream_t travelling as
+ *     void*; NULL = the default stream);
  *   - returns MX_OK or a negative MX_E* code and never throws;
- *   - is re-entrant: there is no mutable global state.
+ *   - allocates nothing, with one exception: the first mx_gemm_nt on a given
+ *     (device, stream) whose shape leaves the last round of tiles mostly empty
+ *     allocates a scratch of 2 x 256 KiB per CU (128 MiB on MI355X) that is kept
+ *     for the life of the process; the call skips that optimisation instead
+ *     when the stream is being captured or the allocation fails;
+ *   - is thread-safe; calls that share a stream share that scratch, which is
+ *     safe because work on one stream runs in order.
  *
  * The reference (KohakUwULLM) has no FFI; each function cites the reference
  * Python/Triton interface it stands in for (paths relative to the reference tree).
@@ -129,6 +135,25 @@ int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const ui
                void *c, int c_dtype, int64_t M, int64_t N, int64_t K,
                int64_t lda, int64_t ldas, int64_t ldb, int64_t ldbs, int64_t ldc,
                int epilogue, void *stream);
+
+/*
+ * Up to any number of independent products C_j = deq(A_j) deq(B_j)^T behind as few
+ * launches as possible (groups of 4 share one launch, the GPU's workgroups divided
+ * among them by work).  Meant for products that are ready at the same time and do not
+ * fill the GPU one by one: DGRAD with WGRAD of a linear layer, the three products that
+ * end a SwiGLU block's backward.  All outputs have dtype c_dtype.  `problems` is a
+ * HOST array, read before the call returns.  Results are those of `count` calls of
+ * mx_gemm_nt with MX_EPI_NONE.
+ * Replaces the back-to-back launches of the reference's backward
+ * (src/kohakuwullm/kernels/mxfp8/linear.py:66-74: dx then dw; models/components/mlp.py:68-73
+ * under autograd).
+ */
+typedef struct mx_gemm_problem {
+    const uint8_t *aq, *a_scale, *bq, *b_scale;
+    void *c;
+    int64_t M, N, K, lda, ldas, ldb, ldbs, ldc;
+} mx_gemm_problem;
+int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *stream);
 
 /*
  * ---- routed experts -------------------------------------------------------------------

@@ -50,7 +50,16 @@ SIGNATURES = {
     "mx_grouped_wgrad_nt": (
         _ci, [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p]),
     "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),
+    "mx_gemm_nt_batch": (_ci, [_p, _ci, _ci, _p]),
 }
+
+
+class GemmProblem(ctypes.Structure):
+    """``mx_gemm_problem`` of the C header."""
+
+    _fields_ = [(n, _p) for n in ("aq", "a_scale", "bq", "b_scale", "c")] + [
+        (n, _i64) for n in ("M", "N", "K", "lda", "ldas", "ldb", "ldbs", "ldc")
+    ]
 
 _lib: ctypes.CDLL | None = None
 

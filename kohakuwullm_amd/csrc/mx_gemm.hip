@@ -3,6 +3,11 @@
 // Semantics: mxfp8_matmul_pq of the reference (src/kohakuwullm/kernels/mxfp8/quantize.py:242-371).
 // The kernel body lives in mx_gemm_core.h; this file supplies the dense problem policy,
 // the slow generic kernel for shapes the tiled kernel does not take, and the C entry point.
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "mx_gemm_core.h"
 
 namespace mx {
@@ -16,21 +21,56 @@ struct DenseArgs {
     int c_vec;
     int accumulate;  // fp32 atomic add into C (split-K)
     int split_k;     // number of K slices; tile ids run over tiles_m * tiles_n * split_k
+    // Even K split of the last, partial round of tiles.  Tile ids [0, dp_tiles) are whole tiles
+    // dealt round-robin; the K stages of the remaining sk_tiles tiles are laid end to end (each
+    // tile padded to KT4 stages) and cut into gridDim.x equal ranges of sk_q stages, one per
+    // workgroup.  A workgroup whose range covers only part of a tile leaves its fp32 partial
+    // in sk_ws; split_reduce_kernel, launched behind the GEMM, adds the pieces and stores C.
+    // (Letting the last workgroup to arrive at a tile add the pieces inside the GEMM was
+    // measured slower: one CU pulls the other pieces at ~40 GB/s, a kernel of its own at TB/s.)
+    int dp_tiles, sk_tiles, sk_q;
+    float *sk_ws;
 };
 
 template <typename S, int CDT>
 struct DenseProblem {
     struct Tile {
         int m0, n0, kt0, kt1;
+        int sk;  // index among the K-split tiles when this unit is one piece of several, else -1
     };
     const DenseArgs p;  // a copy: its fields live in scalar registers, never re-read through a pointer
     int next_id;
     int kb_end;
+    int sk_pos, sk_end;  // this workgroup's remaining range in the K-split stage space
+    const int first, stride;  // this workgroup is number `first` of the `stride` working on the problem
 
-    __device__ DenseProblem(const DenseArgs &args) : p(args), next_id(blockIdx.x), kb_end(args.K >> 5) {}
+    __device__ DenseProblem(const DenseArgs &args, int first_, int stride_)
+        : p(args), next_id(first_), kb_end(args.K >> 5), first(first_), stride(stride_) {
+        const int KT4 = ((p.K >> 7) + 3) & ~3;
+        const int total = p.sk_tiles * KT4;
+        sk_pos = first * p.sk_q;
+        sk_end = sk_pos + p.sk_q < total ? sk_pos + p.sk_q : total;
+    }
 
     __device__ __forceinline__ bool next(Tile &t) {
         const int per_slice = p.tiles_m * p.tiles_n;
+        if (sk_pos < sk_end) {
+            const int KT = p.K >> 7, KT4 = (KT + 3) & ~3;
+            const int local = sk_pos / KT4;
+            const int k0 = sk_pos - local * KT4;
+            const int stop = k0 + (sk_end - sk_pos);
+            int tm, tn;
+            tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn);
+            t.m0 = tm * S::BM;
+            t.n0 = tn * S::BN;
+            t.kt0 = k0;
+            t.kt1 = stop < KT ? stop : KT;
+            t.sk = (k0 == 0 && stop >= KT) ? -1 : local;
+            sk_pos += (stop < KT4 ? stop : KT4) - k0;
+            return true;
+        }
+        t.sk = -1;
+        if (p.sk_tiles && next_id >= p.dp_tiles) return false;
         if (next_id >= per_slice * p.split_k) return false;
         const int slice = next_id / per_slice;
         int tm, tn;
@@ -42,7 +82,7 @@ struct DenseProblem {
         const int per = (((KT + p.split_k - 1) / p.split_k) + 3) & ~3;
         t.kt0 = slice * per < KT ? slice * per : KT;
         t.kt1 = t.kt0 + per < KT ? t.kt0 + per : KT;
-        next_id += gridDim.x;
+        next_id += stride;
         if (t.kt0 == t.kt1) return next(t);  // an empty trailing slice adds nothing
         return true;
     }
@@ -90,7 +130,30 @@ struct DenseProblem {
 
     static constexpr int NST = S::MT * (S::NT / 2) * (CDT == MX_FP32 ? 2 : 1);
 
+    // Slot of workgroup `wg`'s piece of the split tile whose stages start at `begin` in the
+    // split stage space: a workgroup has at most two partial units, the first one continuing
+    // a tile that an earlier workgroup started.
+    __device__ __forceinline__ static v4f *piece_slot(const DenseArgs &p, int wg, int begin) {
+        const int second = begin > wg * p.sk_q ? 1 : 0;
+        return (v4f *)p.sk_ws + (int64_t)(2 * wg + second) * (S::BM * S::BN / 4);
+    }
+
+    // One piece of a K-split tile: the fp32 accumulators go to the workgroup's slot, laid out
+    // [sub-tile][thread] so the stores and the reduction kernel's loads are contiguous.
+    __device__ __forceinline__ void write_piece(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        const int KT4 = ((p.K >> 7) + 3) & ~3;
+        v4f *mine = piece_slot(p, first, t.sk * KT4);
+#pragma unroll
+        for (int i = 0; i < S::MT; i++)
+#pragma unroll
+            for (int j = 0; j < S::NT; j++) mine[(i * S::NT + j) * S::NTHR + L.tid] = acc[i][j];
+    }
+
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        if (t.sk >= 0) {
+            write_piece(t, L, acc);
+            return -1;
+        }
         // Interior tiles of a vector-aligned C store unconditionally: every lane issues NST stores.
         const bool interior = t.m0 + S::BM <= p.M && t.n0 + S::BN <= p.N && p.c_vec && !p.accumulate;
         // sub-tiles (2h, 2h+1) of a lane hold 8 consecutive N starting at b_sub_off(2h) + 8 g
@@ -121,8 +184,59 @@ struct DenseProblem {
 template <typename S, int CDT, bool K512>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    DenseProblem<S, CDT> prob(args);
+    DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
     persistent_gemm<S, K512>(prob, smem);
+}
+
+// Several independent products in one launch.  The workgroups are partitioned among the
+// problems (cu_lo[j] .. cu_lo[j+1]) in proportion to their work, so a product with too few
+// tiles to fill the GPU runs beside the others instead of leaving most of it idle.
+#define MX_BATCH_MAX 4
+struct DenseBatchArgs {
+    DenseArgs prob[MX_BATCH_MAX];
+    int cu_lo[MX_BATCH_MAX + 1];
+    int count;
+};
+
+template <typename S, int CDT, bool K512>
+__global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    int j = 0;
+    while (j + 1 < b.count && (int)blockIdx.x >= b.cu_lo[j + 1]) j++;
+    DenseProblem<S, CDT> prob(b.prob[j], (int)blockIdx.x - b.cu_lo[j], b.cu_lo[j + 1] - b.cu_lo[j]);
+    persistent_gemm<S, K512>(prob, smem);
+}
+
+// Second half of the even K split: each thread owns what one lane of the GEMM epilogue owns
+// (8 consecutive N of one output row of one split tile), adds that piece of every workgroup
+// that worked on the tile, in workgroup order, and stores it.  Tiles a single workgroup
+// covered whole were stored by the GEMM itself.
+template <typename S, int CDT>
+__global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
+    const int KT = p.K >> 7, KT4 = (KT + 3) & ~3;
+    const int local = blockIdx.x / (S::MT * S::NT / 2);
+    const int sub = blockIdx.x % (S::MT * S::NT / 2);
+    const int i = sub / (S::NT / 2), h = sub % (S::NT / 2);
+    const int begin = local * KT4;
+    const int c_lo = begin / p.sk_q, c_hi = (begin + KT - 1) / p.sk_q;
+    if (c_lo == c_hi) return;
+    const int tid = threadIdx.x;
+    v4f lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+    for (int c = c_lo; c <= c_hi; c++) {
+        const v4f *src = DenseProblem<S, CDT>::piece_slot(p, c, begin);
+        lo += src[(i * S::NT + 2 * h) * S::NTHR + tid];
+        hi += src[(i * S::NT + 2 * h + 1) * S::NTHR + tid];
+    }
+    int tm, tn;
+    tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn);
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave / S::WGN, wn = wave % S::WGN;
+    const int m = tm * S::BM + wm * S::WTM + 16 * i + (lane & 15);
+    const int n = tn * S::BN + wn * S::WTN + b_sub_off(2 * h) + 8 * (lane >> 4);
+    if (m < p.M && n < p.N) {
+        const int nvalid = p.N - n < 8 ? p.N - n : 8;
+        store8<CDT>(p.c, (int64_t)m * p.ldc + n, lo, hi, nvalid, p.c_vec != 0);
+    }
 }
 
 // Any K % 32 == 0, any alignment: one thread per output element.  The slow path.
@@ -169,6 +283,40 @@ static int num_cus() {
     return n;
 }
 
+// Scratch of the even K split: two fp32 tile slots per workgroup, kept per (device, stream)
+// for the life of the process so launches on different streams never share it.
+static float *split_scratch(hipStream_t st, int cus, size_t tile_floats) {
+    static std::mutex lock;
+    static std::map<std::pair<int, hipStream_t>, float *> table;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> guard(lock);
+    auto key = std::make_pair(dev, st);
+    auto it = table.find(key);
+    if (it != table.end()) return it->second;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;  // no allocation while the stream is being captured: whole tiles only, this time
+    }
+    float *slots = nullptr;
+    if (hipMalloc((void **)&slots, (size_t)cus * 2 * tile_floats * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        slots = nullptr;
+    }
+    table[key] = slots;  // a failed allocation is remembered: the library keeps working on whole tiles
+    return slots;
+}
+
+// MX_GEMM_SPLIT=0 in the environment keeps every tile whole (for A/B timing and debugging).
+static bool split_mode() {
+    static const bool on = [] {
+        const char *e = std::getenv("MX_GEMM_SPLIT");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 template <typename S, int CDT>
 static int launch_tiled(DenseArgs a, hipStream_t st) {
     a.tiles_m = (a.M + S::BM - 1) / S::BM;
@@ -178,22 +326,51 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
     const bool k512 = a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0;
     const int64_t work = (int64_t)a.tiles_m * a.tiles_n * a.split_k;
     const int cus = num_cus();
-    dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
+    a.dp_tiles = (int)work, a.sk_tiles = 0, a.sk_q = 0, a.sk_ws = nullptr;
+    // The last round of tiles occupies `rest` of the `cus` workgroups for a whole tile time.
+    // Dealing the K stages of those tiles evenly over all workgroups instead saves
+    // (cus - rest) / cus of a tile time and costs an fp32 round trip of every piece plus a
+    // second launch; in units of one K stage, measured: 4 + 0.15 per piece.  Ranges are sk_q
+    // stages, a multiple of 4 (scale fetches are 16-byte aligned) and at least an eighth of a
+    // tile, so no tile is cut into more than 9 pieces.
+    const int rest = (int)(work % cus);
+    const int KT = a.K >> 7, KT4 = (KT + 3) & ~3;
+    if (split_mode() && a.split_k == 1 && !a.accumulate && rest > 0 && KT4 >= 8) {
+        int64_t q = ((int64_t)rest * KT4 + cus - 1) / cus;
+        if (q < KT4 / 8) q = KT4 / 8;
+        q = (q + 3) & ~(int64_t)3;
+        const double pieces = (double)rest * KT4 / q + rest;
+        const double gain = (double)(KT4 - q), cost = 4.0 + 0.15 * pieces;
+        float *slots = gain > 1.25 * cost ? split_scratch(st, cus, (size_t)S::BM * S::BN) : nullptr;
+        if (slots) {
+            a.sk_tiles = rest;
+            a.dp_tiles = (int)work - rest;
+            a.sk_q = (int)q;
+            a.sk_ws = slots;
+        }
+    }
+    dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
     auto kern = k512 ? gemm_nt_kernel<S, CDT, true> : gemm_nt_kernel<S, CDT, false>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
         return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    if (a.sk_tiles)
+        split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * (S::MT * S::NT / 2))), block, 0, st>>>(a);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+static bool tiled_ok(const DenseArgs &a) {
+    const int64_t M = a.M, N = a.N;
+    return a.K % 128 == 0 && aligned(a.aq, 16) && aligned(a.bq, 16) && a.lda % 16 == 0 && a.ldb % 16 == 0 &&
+           aligned(a.as, 4) && aligned(a.bs, 4) && a.ldas % 4 == 0 && a.ldbs % 4 == 0 &&
+           256 * a.lda < (int64_t)0x7FFFFFFF && 256 * a.ldb < (int64_t)0x7FFFFFFF &&
+           ((M + 255) / 256) * ((N + 255) / 256) * a.split_k < 0x7FFFFFFF;
 }
 
 template <int CDT>
 static int gemm_dispatch(DenseArgs a, hipStream_t st) {
     const int64_t M = a.M, N = a.N;
-    const bool tiled_ok = a.K % 128 == 0 && aligned(a.aq, 16) && aligned(a.bq, 16) && a.lda % 16 == 0 &&
-                          a.ldb % 16 == 0 && aligned(a.as, 4) && aligned(a.bs, 4) && a.ldas % 4 == 0 &&
-                          a.ldbs % 4 == 0 && 256 * a.lda < (int64_t)0x7FFFFFFF && 256 * a.ldb < (int64_t)0x7FFFFFFF &&
-                          ((M + 255) / 256) * ((N + 255) / 256) * a.split_k < 0x7FFFFFFF;
-    if (!tiled_ok) {
+    if (!tiled_ok(a)) {
         if (a.accumulate) return MX_EUNSUPPORTED;
         int64_t blocks = (M * N + 255) / 256;
         if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
@@ -205,37 +382,153 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
     return launch_tiled<Big, CDT>(a, st);
 }
 
-extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs, void *c,
-                          int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldas, int64_t ldb,
-                          int64_t ldbs, int64_t ldc, int epilogue, void *stream) {
+// Several products behind one launch, the workgroups shared out among them in groups of 8 (one
+// per XCD, so each problem's tile order keeps its XCD locality).  A group goes, one at a time,
+// to the problem that would otherwise finish last; cost of a problem on n workgroups =
+// rounds of tiles x (K stages + 4 for the tile's prologue and epilogue).
+template <int CDT>
+static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
+    typedef GemmShape<256, 256, 2, 4> S;
+    const int cus = num_cus();
+    const int groups = cus / 8;
+    bool fuse = count > 1 && count <= MX_BATCH_MAX && groups >= count && split_mode();
+    DenseBatchArgs b;
+    int64_t tiles[MX_BATCH_MAX], cost[MX_BATCH_MAX], alone = 0;
+    int share[MX_BATCH_MAX];
+    bool k512 = true;
+    for (int j = 0; j < count && fuse; j++) {
+        DenseArgs &a = probs[j];
+        if (!tiled_ok(a)) {
+            fuse = false;
+            break;
+        }
+        a.tiles_m = (a.M + S::BM - 1) / S::BM;
+        a.tiles_n = (a.N + S::BN - 1) / S::BN;
+        a.c_vec = aligned(a.c, 16) && (a.ldc * (CDT == MX_FP32 ? 4 : 2)) % 16 == 0;
+        a.dp_tiles = a.tiles_m * a.tiles_n, a.sk_tiles = 0, a.sk_q = 0, a.sk_ws = nullptr;
+        k512 = k512 && a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0;
+        tiles[j] = a.dp_tiles;
+        cost[j] = (a.K >> 7) + 4;
+        share[j] = 1;
+        alone += (tiles[j] + cus - 1) / cus * cost[j];
+        b.prob[j] = a;
+    }
+    if (fuse) {
+        auto finish = [&](int j) { return (tiles[j] + 8 * share[j] - 1) / (8 * share[j]) * cost[j]; };
+        for (int left = groups - count; left > 0; left--) {
+            int worst = -1;
+            for (int j = 0; j < count; j++)
+                if (8 * share[j] < tiles[j] && (worst < 0 || finish(j) > finish(worst))) worst = j;
+            if (worst < 0) break;
+            share[worst]++;
+        }
+        int64_t together = 0;
+        b.cu_lo[0] = 0;
+        for (int j = 0; j < count; j++) {
+            together = finish(j) > together ? finish(j) : together;
+            const int64_t wgs = 8 * share[j] < tiles[j] ? 8 * share[j] : tiles[j];
+            b.cu_lo[j + 1] = b.cu_lo[j] + (int)wgs;
+        }
+        fuse = together < alone;
+    }
+    if (!fuse) {
+        for (int j = 0; j < count; j++) {
+            int rc = gemm_dispatch<CDT>(probs[j], st);
+            if (rc != MX_OK) return rc;
+        }
+        return MX_OK;
+    }
+    b.count = count;
+    auto kern = k512 ? gemm_nt_batch_kernel<S, CDT, true> : gemm_nt_batch_kernel<S, CDT, false>;
+    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
+        return MX_ELAUNCH;
+    kern<<<dim3((unsigned)b.cu_lo[count]), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs, void *c,
+                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldas, int64_t ldb, int64_t ldbs, int64_t ldc) {
     if (M < 0 || N < 0 || K < 0 || K % MX_BLOCK || lda < K || ldb < K || ldas < K / MX_BLOCK || ldbs < K / MX_BLOCK ||
         ldc < N || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
         return MX_EINVAL;
+    a.aq = aq, a.as = as, a.bq = bq, a.bs = bs, a.c = c;
+    a.M = (int)M, a.N = (int)N, a.K = (int)K;
+    a.lda = lda, a.ldas = ldas, a.ldb = ldb, a.ldbs = ldbs, a.ldc = ldc;
+    a.accumulate = 0, a.split_k = 1;
+    a.tiles_m = a.tiles_n = a.c_vec = 0;
+    a.dp_tiles = a.sk_tiles = a.sk_q = 0;
+    a.sk_ws = nullptr;
+    return MX_OK;
+}
+
+static int zero_matrix(void *c, int c_dtype, int64_t M, int64_t N, int64_t ldc, hipStream_t st) {
+    const int esz = c_dtype == MX_FP32 ? 4 : 2;
+    hipError_t e = hipMemset2DAsync(c, (size_t)ldc * esz, 0, (size_t)N * esz, (size_t)M, st);
+    return e == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+extern "C" int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *stream) {
+    if (count < 0 || (count > 0 && !problems)) return MX_EINVAL;
+    if (c_dtype != MX_BF16 && c_dtype != MX_FP16 && c_dtype != MX_FP32) return MX_EINVAL;
+    hipStream_t st = (hipStream_t)stream;
+    DenseArgs live[MX_BATCH_MAX];
+    int n = 0;
+    auto flush = [&]() -> int {
+        int rc = MX_OK;
+        if (n) {
+            switch (c_dtype) {
+            case MX_BF16: rc = batch_dispatch<MX_BF16>(live, n, st); break;
+            case MX_FP16: rc = batch_dispatch<MX_FP16>(live, n, st); break;
+            default: rc = batch_dispatch<MX_FP32>(live, n, st); break;
+            }
+        }
+        n = 0;
+        return rc;
+    };
+    for (int j = 0; j < count; j++) {  // validate everything before launching anything
+        const mx_gemm_problem &q = problems[j];
+        DenseArgs probe;
+        int rc = fill_args(probe, q.aq, q.a_scale, q.bq, q.b_scale, q.c, q.M, q.N, q.K, q.lda, q.ldas, q.ldb, q.ldbs, q.ldc);
+        if (rc != MX_OK) return rc;
+    }
+    for (int j = 0; j < count; j++) {
+        const mx_gemm_problem &q = problems[j];
+        if (q.M == 0 || q.N == 0) continue;
+        if (q.K == 0) {
+            int rc = zero_matrix(q.c, c_dtype, q.M, q.N, q.ldc, st);
+            if (rc != MX_OK) return rc;
+            continue;
+        }
+        fill_args(live[n++], q.aq, q.a_scale, q.bq, q.b_scale, q.c, q.M, q.N, q.K, q.lda, q.ldas, q.ldb, q.ldbs, q.ldc);
+        if (n == MX_BATCH_MAX) {
+            int rc = flush();
+            if (rc != MX_OK) return rc;
+        }
+    }
+    return flush();
+}
+
+extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs, void *c,
+                          int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldas, int64_t ldb,
+                          int64_t ldbs, int64_t ldc, int epilogue, void *stream) {
+    DenseArgs a;
+    int rc = fill_args(a, aq, as, bq, bs, c, M, N, K, lda, ldas, ldb, ldbs, ldc);
+    if (rc != MX_OK) return rc;
     const int split_k = epilogue >> 8;  // MX_EPI_SPLIT_K(n)
     const int epi = epilogue & 0xFF;
     if (epi != MX_EPI_NONE && epi != MX_EPI_ACCUMULATE) return MX_EUNSUPPORTED;
     if (epi == MX_EPI_ACCUMULATE && c_dtype != MX_FP32) return MX_EINVAL;
     if (split_k > 1 && epi != MX_EPI_ACCUMULATE) return MX_EINVAL;
+    if (c_dtype != MX_BF16 && c_dtype != MX_FP16 && c_dtype != MX_FP32) return MX_EINVAL;
     if (M == 0 || N == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
-    if (K == 0) {
-        if (epi == MX_EPI_ACCUMULATE) return MX_OK;
-        // An empty contraction is a zero matrix.
-        int esz = c_dtype == MX_FP32 ? 4 : 2;
-        hipError_t e = hipMemset2DAsync(c, (size_t)ldc * esz, 0, (size_t)N * esz, (size_t)M, st);
-        return e == hipSuccess ? MX_OK : MX_ELAUNCH;
-    }
-    DenseArgs a;
-    a.aq = aq, a.as = as, a.bq = bq, a.bs = bs, a.c = c;
-    a.M = (int)M, a.N = (int)N, a.K = (int)K;
-    a.lda = lda, a.ldas = ldas, a.ldb = ldb, a.ldbs = ldbs, a.ldc = ldc;
+    if (K == 0)  // an empty contraction is a zero matrix
+        return epi == MX_EPI_ACCUMULATE ? MX_OK : zero_matrix(c, c_dtype, M, N, ldc, st);
     a.accumulate = epi == MX_EPI_ACCUMULATE;
     a.split_k = split_k > 1 ? split_k : 1;
-    a.tiles_m = a.tiles_n = a.c_vec = 0;
     switch (c_dtype) {
     case MX_BF16: return gemm_dispatch<MX_BF16>(a, st);
     case MX_FP16: return gemm_dispatch<MX_FP16>(a, st);
-    case MX_FP32: return gemm_dispatch<MX_FP32>(a, st);
-    default: return MX_EINVAL;
+    default: return gemm_dispatch<MX_FP32>(a, st);
     }
 }

@@ -235,6 +235,15 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
 
     // Nothing crosses into or out of the stage body, nor from one step of it into the next.
     __builtin_amdgcn_sched_barrier(0);
+    // A fragments are double buffered in registers: the reads for sub-tile i+1 are in
+    // flight while the MFMAs of sub-tile i issue.  LDS reads return in order, so the first
+    // MFMA's operands (A[0], B[0]) are asked for first: it can issue while B[1..] still stream in.
+    v8i af[2];
+    {
+        v4i lo = *(const v4i *)(la + a_lo);
+        v4i hi = *(const v4i *)(la + a_hi);
+        af[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
     v8i bf[S::NT];
 #pragma unroll
     for (int j = 0; j < S::NT; j++) {
@@ -242,14 +251,6 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
         v4i lo = *(const v4i *)(lb + b_lo + o);
         v4i hi = *(const v4i *)(lb + b_hi + o);
         bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-    // A fragments are double buffered in registers: the reads for sub-tile i+1 are in
-    // flight while the MFMAs of sub-tile i issue.
-    v8i af[2];
-    {
-        v4i lo = *(const v4i *)(la + a_lo);
-        v4i hi = *(const v4i *)(la + a_hi);
-        af[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll

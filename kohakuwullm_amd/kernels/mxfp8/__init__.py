@@ -10,6 +10,7 @@ from kohakuwullm_amd.kernels.mxfp8.quantize import (
     E4M3_MAX,
     mxfp8_matmul,
     mxfp8_matmul_pq,
+    mxfp8_matmul_pq_batch,
     quantize_mx,
     quantize_mx_cols,
     quantize_mx_dual,
@@ -20,6 +21,7 @@ __all__ = [
     "E4M3_MAX",
     "mxfp8_matmul",
     "mxfp8_matmul_pq",
+    "mxfp8_matmul_pq_batch",
     "quantize_mx",
     "quantize_mx_cols",
     "quantize_mx_dual",

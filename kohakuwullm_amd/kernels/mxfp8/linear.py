@@ -22,6 +22,7 @@ import torch.nn.functional as F
 from kohakuwullm_amd.kernels.mxfp8.quantize import (
     BLOCK_SCALE,
     mxfp8_matmul_pq,
+    mxfp8_matmul_pq_batch,
     quantize_mx,
     quantize_mx_cols,
     quantize_mx_dual,
@@ -93,7 +94,12 @@ class _MXFP8Linear(torch.autograd.Function):
             dq, ds, dtq, dts = quantize_mx_dual(padded)
             n = ctx.out_features
             # dW (out,in) = dY^T (out,tokens) . (X^T (in,tokens))^T, contraction over tokens.
-            dw = mxfp8_matmul_pq(dtq[:n], dts[:n], x_a, x_b, ctx.compute)
+            wgrad = (dtq[:n], dts[:n], x_a, x_b)
+            if need_dx and ctx.x_dtype == ctx.compute:
+                # few tiles with a long K beside many with a short one: one launch shares the GPU
+                dx, dw = mxfp8_matmul_pq_batch([(dq, ds, wq_d, ws_d), wgrad], ctx.compute)
+                return dx.reshape(*shape[:-1], dx.shape[-1]), dw, None, None, None, None, None
+            dw = mxfp8_matmul_pq(*wgrad, ctx.compute)
         else:
             dq, ds = quantize_mx(padded) if need_dx else (None, None)
             if need_dw:

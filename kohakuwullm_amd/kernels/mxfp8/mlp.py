@@ -19,7 +19,12 @@ import torch
 
 from kohakuwullm_amd import _lib
 from kohakuwullm_amd.kernels.mxfp8.linear import compute_dtype
-from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE, mxfp8_matmul_pq, quantize_mx_dual
+from kohakuwullm_amd.kernels.mxfp8.quantize import (
+    BLOCK_SCALE,
+    mxfp8_matmul_pq,
+    mxfp8_matmul_pq_batch,
+    quantize_mx_dual,
+)
 
 _FP8 = torch.float8_e4m3fn
 
@@ -88,13 +93,25 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         dq, ds, dtq, dts = quantize_mx_dual(d2d)
         dh = mxfp8_matmul_pq(dq, ds, wout_dq, wout_ds, ctx.compute)
         pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu)
-        dx = dw_in = dw_out = None
-        if ctx.needs_input_grad[0]:
-            dx = mxfp8_matmul_pq(pq, ps, win_dq, win_ds, ctx.x_dtype).reshape(*shape[:-1], -1)
-        if ctx.needs_input_grad[1]:
-            dw_in = mxfp8_matmul_pq(ptq, pts, xtq, xts, ctx.compute)
-        if ctx.needs_input_grad[2]:
-            dw_out = mxfp8_matmul_pq(dtq, dts, htq, hts, ctx.compute)
+        # The last three products are independent and none fills the GPU alone (dW has few
+        # tiles with a long K): they go down together and share the GPU by work.
+        wanted = [
+            (pq, ps, win_dq, win_ds) if ctx.needs_input_grad[0] else None,
+            (ptq, pts, xtq, xts) if ctx.needs_input_grad[1] else None,
+            (dtq, dts, htq, hts) if ctx.needs_input_grad[2] else None,
+        ]
+        grads = [None, None, None]
+        if ctx.x_dtype == ctx.compute:
+            live = [i for i, w in enumerate(wanted) if w is not None]
+            for i, g in zip(live, mxfp8_matmul_pq_batch([wanted[i] for i in live], ctx.compute)):
+                grads[i] = g
+        else:
+            for i, w in enumerate(wanted):
+                if w is not None:
+                    grads[i] = mxfp8_matmul_pq(*w, ctx.x_dtype if i == 0 else ctx.compute)
+        dx, dw_in, dw_out = grads
+        if dx is not None:
+            dx = dx.reshape(*shape[:-1], -1)
         return dx, dw_in, dw_out, None, None, None, None
 
 

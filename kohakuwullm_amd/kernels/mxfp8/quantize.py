@@ -12,6 +12,8 @@ Accumulation is fp32 always; the output dtype is the caller's.
 
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from kohakuwullm_amd import _lib
@@ -147,6 +149,48 @@ def mxfp8_matmul_pq(
     if m and n:
         _gemm_nt_into(*tensors, out)
     return out
+
+
+def mxfp8_matmul_pq_batch(problems, out_dtype: torch.dtype = torch.bfloat16) -> list[torch.Tensor]:
+    """``[aq @ bq.T for (aq, a_scale, bq, b_scale) in problems]`` behind as few launches as possible.
+
+    For products that are ready together and do not fill the GPU one by one (DGRAD and WGRAD
+    of one layer): the library divides the GPU among them instead of running them in turn.
+    Same operand contract and same results as :func:`mxfp8_matmul_pq`.
+    """
+    if out_dtype not in _lib.MX_DTYPE:
+        raise ValueError(f"out_dtype={out_dtype} is not one of {tuple(_lib.MX_DTYPE)}")
+    if not problems:
+        return []
+    descs = (_lib.GemmProblem * len(problems))()
+    outs, keep, flops = [], [], 0.0
+    for d, (aq, a_scale, bq, b_scale) in zip(descs, problems):
+        if aq.dim() != 2 or bq.dim() != 2 or aq.shape[1] != bq.shape[1]:
+            raise ValueError(f"contraction mismatch: {tuple(aq.shape)} @ {tuple(bq.shape)}.T")
+        m, k = aq.shape
+        n = bq.shape[0]
+        if k % BLOCK_SCALE:
+            raise ValueError(f"K={k} must be a multiple of {BLOCK_SCALE}")
+        if a_scale.shape != (m, k // BLOCK_SCALE) or b_scale.shape != (n, k // BLOCK_SCALE):
+            raise ValueError(
+                f"scale shapes {tuple(a_scale.shape)}, {tuple(b_scale.shape)} do not match operands "
+                f"{tuple(aq.shape)}, {tuple(bq.shape)}"
+            )
+        _lib.require_gpu(aq, "aq")
+        ts = []
+        for t in (aq, a_scale, bq, b_scale):
+            if t.element_size() != 1:
+                raise ValueError(f"codes and scales must be 1-byte tensors, got {t.dtype}")
+            ts.append(t if t.stride(1) == 1 else t.contiguous())
+        out = torch.empty(m, n, device=aq.device, dtype=out_dtype)
+        keep.append(ts)
+        outs.append(out)
+        flops += 2.0 * m * n * k
+        d.aq, d.a_scale, d.bq, d.b_scale, d.c = (t.data_ptr() for t in (*ts, out))
+        d.M, d.N, d.K = m, n, k
+        d.lda, d.ldas, d.ldb, d.ldbs, d.ldc = ts[0].stride(0), ts[1].stride(0), ts[2].stride(0), ts[3].stride(0), n
+    _lib.invoke("mx_gemm_nt_batch", flops, outs[0], ctypes.addressof(descs), len(problems), _lib.MX_DTYPE[out_dtype])
+    return outs
 
 
 def mxfp8_matmul(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:

@@ -139,6 +139,95 @@ def test_matmul_end_to_end_smoke_config(oracle):
     assert 0.02 < oracle.rel_error(y, exact) < 0.05
 
 
+# Shapes whose last round of tiles fills less than nine tenths of the GPU and whose K is long
+# enough: the library cuts the K range of those tiles evenly over the workgroups and sums fp32
+# pieces in a fixed order.
+SPLIT_SHAPES = [
+    (768, 512, 8192),  # 6 tiles, each cut into 8 pieces
+    (700, 500, 4224),  # ragged edges, K % 512 != 0 (33 stages, padded to 36)
+    (256, 256, 16384),  # a single tile
+    (2048, 1536, 2048),  # 48 tiles
+    (4352, 4096, 1024),  # one whole round of 256 tiles, then 16 more that are split
+]
+
+
+@pytest.mark.parametrize("m,n,k", SPLIT_SHAPES)
+def test_gemm_even_k_split(oracle, m, n, k):
+    aq, as_, bq, bs = _operands(oracle, m, n, k)
+    ref = oracle.gemm_nt(aq, as_, bq, bs)
+    got = _run(aq, as_, bq, bs, torch.float32)
+    assert oracle.rel_error(got, ref) < TOL_FP32
+    # the pieces are added in slot order, never in arrival order: identical bits every time
+    for _ in range(3):
+        assert torch.equal(_run(aq, as_, bq, bs, torch.float32), got)
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run(aq, as_, bq, bs, dtype)
+        assert oracle.rel_error(out, ref) < TOL_BF16
+        # one rounding of the fp32 sum, as without the split
+        assert torch.equal(out, got.to(dtype))
+
+
+BATCHES = [
+    [(512, 384, 1024), (384, 256, 4096), (256, 256, 8192)],  # the shape mix of a backward: short K many tiles, long K few
+    [(300, 200, 640), (64, 64, 96)],  # ragged, and one problem only the generic kernel takes: run in turn
+    [(256, 512, 512)],
+    [(256, 256, 256)] * 6,  # more than one launch's worth
+    [(128, 0, 256), (0, 64, 128), (200, 100, 0), (256, 128, 384)],  # empty problems drop out, K = 0 is a zero matrix
+]
+
+
+@pytest.mark.parametrize("shapes", BATCHES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gemm_batch(oracle, shapes, dtype):
+    f8 = torch.float8_e4m3fn
+    def make(i, m, n, k):
+        if m and n and k:
+            return _operands(oracle, m, n, k, seed=SEED + i)
+        u8 = torch.uint8
+        return torch.zeros(m, k, dtype=u8), torch.zeros(m, k // 32, dtype=u8), torch.zeros(n, k, dtype=u8), torch.zeros(n, k // 32, dtype=u8)
+
+    ops = [make(i, m, n, k) for i, (m, n, k) in enumerate(shapes)]
+    dev_ops = [(aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)) for aq, as_, bq, bs in ops]
+    outs = _mx().mxfp8_matmul_pq_batch(dev_ops, dtype)
+    assert len(outs) == len(shapes)
+    for (m, n, k), op, dop, out in zip(shapes, ops, dev_ops, outs):
+        assert out.shape == (m, n) and out.dtype == dtype
+        if m == 0 or n == 0:
+            continue
+        if k == 0:
+            assert not out.any()
+            continue
+        ref = oracle.gemm_nt(*op)
+        assert oracle.rel_error(out.cpu(), ref) < (TOL_FP32 if dtype == torch.float32 else TOL_BF16)
+        # a launch of its own may cut K differently (few tiles, long K): same sum up to fp32 reassociation
+        alone = _mx().mxfp8_matmul_pq(*dop, dtype)
+        assert oracle.rel_error(out.cpu(), alone.double().cpu()) < (1e-6 if dtype == torch.float32 else 1e-3)
+    with pytest.raises(ValueError):
+        _mx().mxfp8_matmul_pq_batch([(dev_ops[0][0], dev_ops[0][1], dev_ops[0][2][:, :32], dev_ops[0][3])], dtype)
+    assert _mx().mxfp8_matmul_pq_batch([], dtype) == []
+
+
+def test_gemm_split_k_accumulate(oracle):
+    """The caller-driven split: fp32 atomic accumulation into a C the caller zeroed (or holds a bias in)."""
+    from kohakuwullm_amd import _lib
+
+    m, n, k = 300, 520, 4096
+    aq, as_, bq, bs = _operands(oracle, m, n, k)
+    ref = oracle.gemm_nt(aq, as_, bq, bs)
+    f8 = torch.float8_e4m3fn
+    a, sa, b, sb = aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)
+    base = torch.randn(m, n, device=DEV)
+    for split in (1, 4, 7):
+        c = base.clone()
+        _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(),
+                    _lib.MX_DTYPE[torch.float32], m, n, k, k, k // 32, k, k // 32, n, 1 | (split << 8))
+        assert oracle.rel_error((c - base).cpu(), ref) < TOL_FP32, split
+    c16 = torch.zeros(m, n, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):  # accumulation is fp32 only
+        _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c16.data_ptr(),
+                    _lib.MX_DTYPE[torch.bfloat16], m, n, k, k, k // 32, k, k // 32, n, 1)
+
+
 def test_gemm_errors():
     mx = _mx()
     f8 = torch.float8_e4m3fn
