@@ -103,14 +103,15 @@ struct DenseProblem {
         }
 #pragma unroll
         for (int q = 0; q < S::QB; q++) {
-            int row = dma_row<S>(L, q);
-            int chunk = (L.lane & 7) ^ swz_b(row);
-            int grow = row < nrem ? row : nrem - 1;
+            int row = dma_row<S>(L, q);  // LDS row; it holds B row b_row_of_lds(row) of the tile
+            int chunk = (L.lane & 7) ^ swz_a(row);
+            int brow = b_row_of_lds<S>(row);
+            int grow = brow < nrem ? brow : nrem - 1;
             c.b_voff[q] = (uint32_t)(grow * p.ldb) + chunk * 16;
         }
         auto srow = [&](int r) -> const uint8_t * {
             if (r < S::BM) return p.as + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.ldas;
-            r -= S::BM;
+            r = b_row_of_lds<S>(r - S::BM);
             return p.bs + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldbs;
         };
         c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
@@ -123,12 +124,13 @@ struct DenseProblem {
             const int mrem = p.M - t.m0;
             return p.aq + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.lda;
         }
-        r -= S::BM;
+        r = b_row_of_lds<S>(r - S::BM);
         const int nrem = p.N - t.n0;
         return p.bq + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldb;
     }
 
-    static constexpr int NST = S::MT * (S::NT / 2) * (CDT == MX_FP32 ? 2 : 1);
+    static_assert(S::LANES_N, "the dense kernels use the layout that puts neighbouring lanes on neighbouring N");
+    static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
     // Slot of workgroup `wg`'s piece of the split tile whose stages start at `begin` in the
     // split stage space: a workgroup has at most two partial units, the first one continuing
@@ -156,23 +158,25 @@ struct DenseProblem {
         }
         // Interior tiles of a vector-aligned C store unconditionally: every lane issues NST stores.
         const bool interior = t.m0 + S::BM <= p.M && t.n0 + S::BN <= p.N && p.c_vec && !p.accumulate;
-        // sub-tiles (2h, 2h+1) of a lane hold 8 consecutive N starting at b_sub_off(2h) + 8 g
+        // component v of a lane's 8 sub-tiles (i, 0..7): row 16 i + 4 g + v, 8 consecutive N from 8 r16
+        const int n = t.n0 + L.wn * S::WTN + 8 * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
-            const int m = t.m0 + L.wm * S::WTM + 16 * i + L.r16;
 #pragma unroll
-            for (int h = 0; h < S::NT / 2; h++) {
-                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+            for (int v = 0; v < 4; v++) {
+                const int m = t.m0 + L.wm * S::WTM + 16 * i + 4 * L.g + v;
                 const int64_t off = (int64_t)m * p.ldc + n;
+                const v4f lo = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+                const v4f hi = {acc[i][4][v], acc[i][5][v], acc[i][6][v], acc[i][7][v]};
                 if (interior) {
-                    store8<CDT>(p.c, off, acc[i][2 * h], acc[i][2 * h + 1], 8, true);
+                    store8<CDT>(p.c, off, lo, hi, 8, true);
                 } else if (m < p.M && n < p.N) {
                     const int nvalid = p.N - n < 8 ? p.N - n : 8;
                     if (CDT == MX_FP32 && p.accumulate) {
                         float *dst = (float *)p.c + off;
-                        for (int e = 0; e < 8 && e < nvalid; e++) atomicAdd(dst + e, e < 4 ? acc[i][2 * h][e] : acc[i][2 * h + 1][e - 4]);
+                        for (int e = 0; e < 8 && e < nvalid; e++) atomicAdd(dst + e, e < 4 ? lo[e] : hi[e - 4]);
                     } else {
-                        store8<CDT>(p.c, off, acc[i][2 * h], acc[i][2 * h + 1], nvalid, p.c_vec != 0);
+                        store8<CDT>(p.c, off, lo, hi, nvalid, p.c_vec != 0);
                     }
                 }
             }
@@ -208,34 +212,40 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b
 }
 
 // Second half of the even K split: each thread owns what one lane of the GEMM epilogue owns
-// (8 consecutive N of one output row of one split tile), adds that piece of every workgroup
+// for one i (4 rows x 8 consecutive N of one split tile), adds that piece of every workgroup
 // that worked on the tile, in workgroup order, and stores it.  Tiles a single workgroup
 // covered whole were stored by the GEMM itself.
 template <typename S, int CDT>
 __global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
     const int KT = p.K >> 7, KT4 = (KT + 3) & ~3;
-    const int local = blockIdx.x / (S::MT * S::NT / 2);
-    const int sub = blockIdx.x % (S::MT * S::NT / 2);
-    const int i = sub / (S::NT / 2), h = sub % (S::NT / 2);
+    const int local = blockIdx.x / S::MT;
+    const int i = blockIdx.x % S::MT;
     const int begin = local * KT4;
     const int c_lo = begin / p.sk_q, c_hi = (begin + KT - 1) / p.sk_q;
     if (c_lo == c_hi) return;
     const int tid = threadIdx.x;
-    v4f lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+    v4f sum[S::NT];
+#pragma unroll
+    for (int j = 0; j < S::NT; j++) sum[j] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int c = c_lo; c <= c_hi; c++) {
         const v4f *src = DenseProblem<S, CDT>::piece_slot(p, c, begin);
-        lo += src[(i * S::NT + 2 * h) * S::NTHR + tid];
-        hi += src[(i * S::NT + 2 * h + 1) * S::NTHR + tid];
+#pragma unroll
+        for (int j = 0; j < S::NT; j++) sum[j] += src[(i * S::NT + j) * S::NTHR + tid];
     }
     int tm, tn;
     tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn);
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WGN, wn = wave % S::WGN;
-    const int m = tm * S::BM + wm * S::WTM + 16 * i + (lane & 15);
-    const int n = tn * S::BN + wn * S::WTN + b_sub_off(2 * h) + 8 * (lane >> 4);
-    if (m < p.M && n < p.N) {
-        const int nvalid = p.N - n < 8 ? p.N - n : 8;
-        store8<CDT>(p.c, (int64_t)m * p.ldc + n, lo, hi, nvalid, p.c_vec != 0);
+    const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int m = tm * S::BM + wm * S::WTM + 16 * i + 4 * (lane >> 4) + v;
+        if (m < p.M && n < p.N) {
+            const int nvalid = p.N - n < 8 ? p.N - n : 8;
+            const v4f lo = {sum[0][v], sum[1][v], sum[2][v], sum[3][v]};
+            const v4f hi = {sum[4][v], sum[5][v], sum[6][v], sum[7][v]};
+            store8<CDT>(p.c, (int64_t)m * p.ldc + n, lo, hi, nvalid, p.c_vec != 0);
+        }
     }
 }
 
@@ -355,9 +365,12 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
         return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     if (a.sk_tiles)
-        split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * (S::MT * S::NT / 2))), block, 0, st>>>(a);
+        split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * S::MT)), block, 0, st>>>(a);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
+
+// 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
+typedef GemmShape<256, 256, 4, 2, true> DenseShape;
 
 static bool tiled_ok(const DenseArgs &a) {
     const int64_t M = a.M, N = a.N;
@@ -378,8 +391,7 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
                                                                                   a.lda, a.ldas, a.ldb, a.ldbs, a.ldc);
         return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
     }
-    typedef GemmShape<256, 256, 2, 4> Big;
-    return launch_tiled<Big, CDT>(a, st);
+    return launch_tiled<DenseShape, CDT>(a, st);
 }
 
 // Several products behind one launch, the workgroups shared out among them in groups of 8 (one
@@ -388,7 +400,7 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
 // rounds of tiles x (K stages + 4 for the tile's prologue and epilogue).
 template <int CDT>
 static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
-    typedef GemmShape<256, 256, 2, 4> S;
+    typedef DenseShape S;
     const int cus = num_cus();
     const int groups = cus / 8;
     bool fuse = count > 1 && count <= MX_BATCH_MAX && groups >= count && split_mode();
