@@ -200,6 +200,22 @@ int mx_experts_scatter_gemm(const uint8_t *aq, const uint8_t *as, int64_t a_rows
                             void *out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K, void *stream);
 
 /*
+ * The same combine without atomics: out (T,N)[t] = sum over k < top_k of
+ * scale(t,k) * y[pos(t,k)], where y (M,N) holds one 16-bit row per sorted position (the
+ * output of mx_grouped_gemm_nt), pair t*top_k + k sits at the sorted position m with
+ * order[m] == t*top_k + k and m < offsets[E] (a pair found nowhere was dropped and adds
+ * nothing), and scale = gate[pair] (NULL: 1).  fp32 sum in k order, one rounding: one writer
+ * per element, bitwise reproducible.  `inv` is caller-provided scratch of T*top_k int32.
+ * Every element of out is written; out need not be zeroed.
+ * Stands in for the tl.atomic_add epilogues of _experts_gemm2 (experts.py:138-222) and
+ * _experts_gemm1_dgrad (experts_bwd.py:167-247) when order is the reference's pair index
+ * (moe.py: token_of = order // top_k).
+ */
+int mx_experts_combine(const void *y, int64_t ldy, const int32_t *order, const int32_t *offsets, int64_t E,
+                       const void *gate, int gate_dtype, int32_t *inv, int64_t T, int64_t top_k,
+                       void *out, int dtype, int64_t ldo, int64_t M, int64_t N, void *stream);
+
+/*
  * DGRAD through GEMM2, the combine and SwiGLU at once: acc = dq[token_of[m]] . w_out_dgrad[e]^T
  * (M,H); dgate[order[m]] += <acc, dequant(hq,hs)[m]> (fp32 atomics, caller-zeroed);
  * dh = acc * gate[order[m]]; SwiGLU backward from the stored pre; dpre (M,2H) stored in

@@ -110,14 +110,18 @@ __device__ __forceinline__ void atomic_add2(void *base, int64_t off, float a, fl
 
 __device__ __forceinline__ float sigmoid_f(float x) { return __fdividef(1.0f, 1.0f + __expf(-x)); }
 
-// max over the four lanes that share an output row (l, l^16, l^32, l^48)
-__device__ __forceinline__ float row_group_max(float a) {
-    a = fmaxf(a, __shfl_xor(a, 16, 64));
-    return fmaxf(a, __shfl_xor(a, 32, 64));
+// Reductions over neighbouring lanes.  A lane owns 8 (GEMM1: 4) consecutive channels of a row
+// and its neighbours own the next ones, so a 32-channel MX block is a quad (GEMM1: 8 lanes)
+// and a wave's whole row segment is a 16-lane DPP row.
+__device__ __forceinline__ float oct_max(float a) {
+    a = quad_max(a);
+    return fmaxf(a, __shfl_xor(a, 4, 64));
 }
-__device__ __forceinline__ float row_group_sum(float a) {
-    a += __shfl_xor(a, 16, 64);
-    return a + __shfl_xor(a, 32, 64);
+__device__ __forceinline__ float row16_sum(float a) {
+    a += __shfl_xor(a, 1, 64);
+    a += __shfl_xor(a, 2, 64);
+    a += __shfl_xor(a, 4, 64);
+    return a + __shfl_xor(a, 8, 64);
 }
 
 template <typename S, int MODE, int CDT>
@@ -131,10 +135,14 @@ struct GroupedProblem {
     // incremental tile_owner: experts [0, scan_e) own row tiles [0, scan_tiles)
     int scan_e, scan_tiles;
 
-    // GEMM1 packs 32 gate + 32 value rows of w_in into each wave's 64-row slice of the B tile,
-    // so a tile spans BN/2 hidden units.
+    // Accumulator layout (GemmShape LANES_N): lane (r16, g) holds, for sub-tile (i, j) and
+    // register v, row 16 i + 4 g + v of the wave's 64 rows and column 8 r16 + j of its 128.
+    // GEMM1 fills each wave's 128-row slice of the B tile with 64 gate rows (sub-tiles 0-3) and
+    // the 64 value rows of the same hidden units (sub-tiles 4-7), so a tile spans BN/2 hidden
+    // units and a lane owns 4 consecutive ones, gate and value.
+    static_assert(S::LANES_N, "the expert kernels use the layout that puts neighbouring lanes on neighbouring N");
     static constexpr int N_PER_TILE = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
-    static constexpr int NST = S::MT * (S::NT / 2) * (CDT == MX_FP32 ? 2 : 1);
+    static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
     __device__ GroupedProblem(const GroupedArgs &a)
         : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0) {}
@@ -187,15 +195,16 @@ struct GroupedProblem {
         pos = pos < t.end ? pos : t.end - 1;
         return p.index ? p.index[pos] : pos;
     }
-    // row of the expert's weight matrix behind B tile row r
+    // row of the expert's weight matrix kept in LDS row r of the B tile
     __device__ __forceinline__ int b_src_row(const Tile &t, int r) const {
         if (MODE == MODE_GEMM1) {
-            const int slice = r >> 6, within = r & 63;
-            int h = t.n0 + slice * 32 + (within & 31);
+            const int slice = r / S::WTN, within = r % S::WTN;
+            const int j = within >> 4, rr = within & 15;
+            int h = t.n0 + slice * (S::WTN / 2) + 4 * rr + (j & 3);
             h = h < p.N ? h : p.N - 1;
-            return within < 32 ? h : p.N + h;
+            return j < 4 ? h : p.N + h;
         }
-        const int n = t.n0 + r;
+        const int n = t.n0 + b_row_of_lds<S>(r);
         return n < p.N ? n : p.N - 1;
     }
 
@@ -213,7 +222,7 @@ struct GroupedProblem {
 #pragma unroll
         for (int q = 0; q < S::QB; q++) {
             const int row = dma_row<S>(L, q);
-            c.b_voff[q] = (uint32_t)((int64_t)b_src_row(t, row) * p.ldw) + (((L.lane & 7) ^ swz_b(row)) << 4);
+            c.b_voff[q] = (uint32_t)((int64_t)b_src_row(t, row) * p.ldw) + (((L.lane & 7) ^ swz_a(row)) << 4);
         }
         auto srow = [&](int r) -> const uint8_t * {
             if (r < S::BM) return p.xs + (int64_t)a_src_row(t, r) * p.ldxs;
@@ -235,67 +244,65 @@ struct GroupedProblem {
         return epilogue_dgrad2(t, L, acc);
     }
 
+    // sorted row of (i, v) for this lane
+    __device__ __forceinline__ int row_of(const Tile &t, const Lane &L, int i, int v) const {
+        return t.row0 + L.wm * S::WTM + 16 * i + 4 * L.g + v;
+    }
+
     // ---- PLAIN: rows of the expert's range are written, nothing else is touched
     __device__ __forceinline__ int epilogue_plain(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
         const bool interior = t.row0 + S::BM <= t.end && t.n0 + S::BN <= p.N && p.out_vec;
+        const int n = t.n0 + L.wn * S::WTN + 8 * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
-            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
 #pragma unroll
-            for (int h = 0; h < S::NT / 2; h++) {
-                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+            for (int v = 0; v < 4; v++) {
+                const int m = row_of(t, L, i, v);
                 const int64_t off = (int64_t)m * p.ldo + n;
-                if (interior) store8<CDT>(p.out, off, acc[i][2 * h], acc[i][2 * h + 1], 8, true);
-                else if (m < t.end && n < p.N)
-                    store8<CDT>(p.out, off, acc[i][2 * h], acc[i][2 * h + 1], p.N - n < 8 ? p.N - n : 8, p.out_vec != 0);
+                const v4f lo = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+                const v4f hi = {acc[i][4][v], acc[i][5][v], acc[i][6][v], acc[i][7][v]};
+                if (interior) store8<CDT>(p.out, off, lo, hi, 8, true);
+                else if (m < t.end && n < p.N) store8<CDT>(p.out, off, lo, hi, p.N - n < 8 ? p.N - n : 8, p.out_vec != 0);
             }
         }
         return interior ? NST : -1;
     }
 
-    // ---- GEMM1: sub-tiles (4q, 4q+1) are gate, (4q+2, 4q+3) value of the same 8 hidden units
+    // ---- GEMM1: sub-tiles 0-3 are gate, 4-7 value of the lane's 4 hidden units
     __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        const int hblock = t.n0 + L.wn * (S::WTN / 2) + 32 * (L.r16 >> 3);  // the 32 hidden units of 8 lanes
+        const int h = t.n0 + L.wn * (S::WTN / 2) + 4 * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
-            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
-            const bool row_ok = m < t.end;
 #pragma unroll
-            for (int q = 0; q < S::NT / 4; q++) {
-                // this wave's 32 hidden units of slice (wn, q); the lane owns 8 of them
-                const int hblock = t.n0 + (L.wn * (S::NT / 4) + q) * 32;
-                const int h = hblock + 8 * L.g;
-                const bool ok = row_ok && hblock < p.N;  // H % 32 == 0: a block is in or out
-                float gv[8], vv[8];
-                uint32_t gp[4], vp[4];
+            for (int v = 0; v < 4; v++) {
+                const int m = row_of(t, L, i, v);
+                const bool ok = m < t.end && hblock < p.N;  // H % 32 == 0: a block is in or out
+                float gv[4], vv[4];
+                uint32_t gp[2], vp[2];
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    gv[e] = acc[i][4 * q][e], gv[4 + e] = acc[i][4 * q + 1][e];
-                    vv[e] = acc[i][4 * q + 2][e], vv[4 + e] = acc[i][4 * q + 3][e];
-                }
+                for (int e = 0; e < 4; e++) gv[e] = acc[i][e][v], vv[e] = acc[i][4 + e][v];
                 // h is rounded to the storage dtype before the activation, so the backward
                 // differentiates the function the forward evaluated (experts.py:116-119)
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
+                for (int e = 0; e < 2; e++) {
                     round_pair<CDT>(gv[2 * e], gv[2 * e + 1], gp[e]);
                     round_pair<CDT>(vv[2 * e], vv[2 * e + 1], vp[e]);
                 }
                 if (ok && p.pre) {
                     uint16_t *pp = (uint16_t *)p.pre + (int64_t)m * p.ldpre + h;
-                    *(v4i *)pp = v4i{(int)gp[0], (int)gp[1], (int)gp[2], (int)gp[3]};
-                    *(v4i *)(pp + p.N) = v4i{(int)vp[0], (int)vp[1], (int)vp[2], (int)vp[3]};
+                    *(v2i *)pp = v2i{(int)gp[0], (int)gp[1]};
+                    *(v2i *)(pp + p.N) = v2i{(int)vp[0], (int)vp[1]};
                 }
-                float a[8];
+                float a[4];
 #pragma unroll
-                for (int e = 0; e < 8; e++) a[e] = gv[e] * sigmoid_f(gv[e]) * vv[e];
-                const float amax = row_group_max(amax8(a));
+                for (int e = 0; e < 4; e++) a[e] = gv[e] * sigmoid_f(gv[e]) * vv[e];
+                const float amax = oct_max(fmaxf(fmaxf(fabsf(a[0]), fabsf(a[1])), fmaxf(fabsf(a[2]), fabsf(a[3]))));
                 const uint32_t byte = scale_byte(amax);
                 const float inv = inv_scale(byte);
                 if (ok) {
-                    v2i codes;
-                    codes[0] = (int)pack4_e4m3(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv);
-                    codes[1] = (int)pack4_e4m3(a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
-                    *(v2i *)(p.hq + (int64_t)m * p.ldhq + h) = codes;
-                    if (L.g == 0) p.hs[(int64_t)m * p.ldhs + (hblock >> 5)] = (uint8_t)byte;
+                    *(uint32_t *)(p.hq + (int64_t)m * p.ldhq + h) = pack4_e4m3(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv);
+                    if ((L.r16 & 7) == 0) p.hs[(int64_t)m * p.ldhs + (hblock >> 5)] = (uint8_t)byte;
                 }
             }
         }
@@ -304,26 +311,21 @@ struct GroupedProblem {
 
     // ---- SCATTER: out[token(m)] += scale(m) * acc, packed 16-bit (or fp32) atomics
     __device__ __forceinline__ int epilogue_scatter(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        const int n = t.n0 + L.wn * S::WTN + 8 * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
-            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
-            if (m >= t.end) continue;
-            const int target = p.token_of[m];
-            float scale = 1.0f;
-            if (p.gate) scale = p.gate_f32 ? ((const float *)p.gate)[p.order[m]] : load_act<CDT>(p.gate, p.order[m]);
 #pragma unroll
-            for (int h = 0; h < S::NT / 2; h++) {
-                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+            for (int v = 0; v < 4; v++) {
+                const int m = row_of(t, L, i, v);
+                if (m >= t.end) continue;
+                const int target = p.token_of[m];
+                float scale = 1.0f;
+                if (p.gate) scale = p.gate_f32 ? ((const float *)p.gate)[p.order[m]] : load_act<CDT>(p.gate, p.order[m]);
                 const int64_t off = (int64_t)target * p.ldo + n;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const float a = (e < 2 ? acc[i][2 * h][2 * e] : acc[i][2 * h + 1][2 * e - 4]) * scale;
-                    const float b = (e < 2 ? acc[i][2 * h][2 * e + 1] : acc[i][2 * h + 1][2 * e - 3]) * scale;
-                    if (n + 2 * e + 1 < p.N) atomic_add2<CDT>(p.out, off + 2 * e, a, b);
-                    else if (n + 2 * e < p.N) {
-                        // odd tail: a lone element (N % 2 == 1 never happens for 32-multiples, kept for safety)
-                        atomic_add2<CDT>(p.out, off + 2 * e - 1, 0.0f, a);
-                    }
+                    const float a = acc[i][2 * e][v] * scale, b = acc[i][2 * e + 1][v] * scale;
+                    if (n + 2 * e + 1 < p.N) atomic_add2<CDT>(p.out, off + 2 * e, a, b);  // N is even
                 }
             }
         }
@@ -333,23 +335,22 @@ struct GroupedProblem {
     // ---- DGRAD2: the accumulator dout[t] . W_out is consumed three ways in registers
     __device__ __forceinline__ int epilogue_dgrad2(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
         const int H = p.N;
+        const int hblock = t.n0 + L.wn * S::WTN + 32 * (L.r16 >> 2);  // the 32 hidden units of a quad
+        const int h = t.n0 + L.wn * S::WTN + 8 * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
-            const int m = t.row0 + L.wm * S::WTM + 16 * i + L.r16;
-            const bool row_ok = m < t.end;
-            const int mm = row_ok ? m : t.end - 1;
-            const int pair = p.order[mm];
-            const float gate = p.gate_f32 ? ((const float *)p.gate)[pair] : load_act<CDT>(p.gate, pair);
-            float dot = 0.0f;
 #pragma unroll
-            for (int hh = 0; hh < S::NT / 2; hh++) {
-                const int hblock = t.n0 + L.wn * S::WTN + b_sub_off(2 * hh);  // 32 hidden units of the 4 lanes
-                const int h = hblock + 8 * L.g;
+            for (int v = 0; v < 4; v++) {
+                const int m = row_of(t, L, i, v);
+                const bool row_ok = m < t.end;
+                const int mm = row_ok ? m : t.end - 1;
+                const int pair = p.order[mm];
+                const float gate = p.gate_f32 ? ((const float *)p.gate)[pair] : load_act<CDT>(p.gate, pair);
                 const bool ok = row_ok && hblock < H;
                 float a[8];
 #pragma unroll
-                for (int e = 0; e < 4; e++) a[e] = acc[i][2 * hh][e], a[4 + e] = acc[i][2 * hh + 1][e];
-                float dg[8], dv[8];
+                for (int e = 0; e < 8; e++) a[e] = acc[i][e][v];
+                float dg[8], dv[8], dot = 0.0f;
                 if (ok) {
                     // h read back from its fp8 copy: the forward multiplied those values
                     const v2i hc = *(const v2i *)(p.hq + (int64_t)mm * p.ldhq + h);
@@ -376,8 +377,8 @@ struct GroupedProblem {
                     for (int e = 0; e < 8; e++) dg[e] = dv[e] = 0.0f;
                 }
                 // both halves: store dpre in the storage dtype, quantize from the fp32 values
-                const float amax_g = row_group_max(amax8(dg));
-                const float amax_v = row_group_max(amax8(dv));
+                const float amax_g = quad_max(amax8(dg));
+                const float amax_v = quad_max(amax8(dv));
                 const uint32_t bg = scale_byte(amax_g), bv = scale_byte(amax_v);
                 const float ig = inv_scale(bg), iv = inv_scale(bv);
                 if (ok) {
@@ -401,20 +402,71 @@ struct GroupedProblem {
                     uint8_t *qp = p.dpq + (int64_t)m * p.lddpq + h;
                     *(v2i *)qp = cg;
                     *(v2i *)(qp + H) = cv;
-                    if (L.g == 0) {
+                    if ((L.r16 & 3) == 0) {
                         uint8_t *sp = p.dps + (int64_t)m * p.lddps + (hblock >> 5);
                         sp[0] = (uint8_t)bg;
                         sp[H >> 5] = (uint8_t)bv;
                     }
                 }
+                // the dot product over the expert width is split across lanes, waves and N tiles
+                dot = row16_sum(dot);
+                if (row_ok && L.r16 == 0) atomicAdd(p.dgate + pair, dot);
             }
-            // the dot product over the expert width is split across lanes, waves and N tiles
-            dot = row_group_sum(dot);
-            if (row_ok && L.g == 0) atomicAdd(p.dgate + pair, dot);
         }
         return -1;
     }
 };
+
+// ---- combine: out[t] = sum_k scale(t,k) * y[pos(t,k)] ---------------------------------------------
+// The scatter-add of the routed rows back to their tokens, as a gather: pair p = t * top_k + k
+// sits at sorted position inv[p] (or nowhere: -1, a dropped pair).  One writer per output
+// element, fp32 sum in slot order, one rounding: deterministic, and an order of magnitude
+// faster than 16-bit atomics for top_k rows per token.
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t *dst, int64_t n, int32_t value) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = value;
+}
+
+__global__ __launch_bounds__(256) void invert_order_kernel(const int32_t *__restrict__ order,
+                                                            const int32_t *__restrict__ offsets, int E, int64_t M,
+                                                            int64_t pairs, int32_t *__restrict__ inv) {
+    const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (m >= M || m >= offsets[E]) return;  // rows past the last expert belong to nobody
+    const int64_t p = order[m];
+    if (p >= 0 && p < pairs) inv[p] = (int32_t)m;
+}
+
+template <int CDT>
+__global__ __launch_bounds__(256) void combine_kernel(const uint16_t *__restrict__ y, int64_t ldy,
+                                                       const int32_t *__restrict__ inv, const void *__restrict__ gate,
+                                                       int gate_f32, int top_k, uint16_t *__restrict__ out, int64_t ldo,
+                                                       int64_t T, int N8) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t t = idx / N8;
+    const int c = (int)(idx - t * N8) * 8;
+    if (t >= T) return;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = 0.0f;
+    for (int k = 0; k < top_k; k++) {
+        const int64_t pair = t * top_k + k;
+        const int pos = inv[pair];
+        if (pos < 0) continue;
+        float scale = 1.0f;
+        if (gate) scale = gate_f32 ? ((const float *)gate)[pair] : load_act<CDT>(gate, pair);
+        float v[8];
+        unpack8<CDT>(*(const v4i *)(y + (int64_t)pos * ldy + c), v);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += scale * v[e];
+    }
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float a = acc[2 * e], b = acc[2 * e + 1];
+        round_pair<CDT>(a, b, w[e]);
+    }
+    *(v4i *)(out + t * ldo + c) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+}
 
 template <typename S, int MODE, int CDT, bool K512>
 __global__ __launch_bounds__(S::NTHR) void grouped_kernel(GroupedArgs args) {
@@ -475,7 +527,7 @@ struct WgradProblem {
     };
     const WgradArgs p;
     int next_id, kb_end, scan_e, scan_tiles;
-    static constexpr int NST = S::MT * (S::NT / 2) * (CDT == MX_FP32 ? 2 : 1);
+    static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
     __device__ WgradProblem(const WgradArgs &a) : p(a), next_id(blockIdx.x), kb_end(a.KB), scan_e(0), scan_tiles(0) {}
 
@@ -533,11 +585,12 @@ struct WgradProblem {
 #pragma unroll
         for (int q = 0; q < S::QB; q++) {
             const int row = dma_row<S>(L, q);
-            c.b_voff[q] = (uint32_t)((int64_t)(row < nrem ? row : nrem - 1) * p.ldb) + (((L.lane & 7) ^ swz_b(row)) << 4);
+            const int brow = b_row_of_lds<S>(row);
+            c.b_voff[q] = (uint32_t)((int64_t)(brow < nrem ? brow : nrem - 1) * p.ldb) + (((L.lane & 7) ^ swz_a(row)) << 4);
         }
         auto srow = [&](int r) -> const uint8_t * {
             if (r < S::BM) return p.as + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.ldas;
-            r -= S::BM;
+            r = b_row_of_lds<S>(r - S::BM);
             return p.bs + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldbs;
         };
         c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
@@ -546,23 +599,24 @@ struct WgradProblem {
 
     __device__ __forceinline__ const uint8_t *line(const Tile &t, int r) const {
         if (r < S::BM) return p.aq + (int64_t)(t.m0 + r < p.N ? t.m0 + r : p.N - 1) * p.lda;
-        r -= S::BM;
+        r = b_row_of_lds<S>(r - S::BM);
         return p.bq + (int64_t)(t.n0 + r < p.Kout ? t.n0 + r : p.Kout - 1) * p.ldb;
     }
 
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
         const bool interior = t.m0 + S::BM <= p.N && t.n0 + S::BN <= p.Kout && p.c_vec;
         const int64_t base = (int64_t)t.expert * p.stride_dwe;
+        const int n = t.n0 + L.wn * S::WTN + 8 * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
-            const int m = t.m0 + L.wm * S::WTM + 16 * i + L.r16;
 #pragma unroll
-            for (int h = 0; h < S::NT / 2; h++) {
-                const int n = t.n0 + L.wn * S::WTN + b_sub_off(2 * h) + 8 * L.g;
+            for (int v = 0; v < 4; v++) {
+                const int m = t.m0 + L.wm * S::WTM + 16 * i + 4 * L.g + v;
                 const int64_t off = base + (int64_t)m * p.lddw + n;
-                if (interior) store8<CDT>(p.dw, off, acc[i][2 * h], acc[i][2 * h + 1], 8, true);
-                else if (m < p.N && n < p.Kout)
-                    store8<CDT>(p.dw, off, acc[i][2 * h], acc[i][2 * h + 1], p.Kout - n < 8 ? p.Kout - n : 8, p.c_vec != 0);
+                const v4f lo = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+                const v4f hi = {acc[i][4][v], acc[i][5][v], acc[i][6][v], acc[i][7][v]};
+                if (interior) store8<CDT>(p.dw, off, lo, hi, 8, true);
+                else if (m < p.N && n < p.Kout) store8<CDT>(p.dw, off, lo, hi, p.Kout - n < 8 ? p.Kout - n : 8, p.c_vec != 0);
             }
         }
         return interior ? NST : -1;
@@ -589,7 +643,8 @@ static int num_cus() {
     return n;
 }
 
-typedef GemmShape<256, 256, 2, 4> Big;
+// 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
+typedef GemmShape<256, 256, 4, 2, true> Big;
 
 static bool tiled_ok(const GroupedArgs &a, int64_t a_rows) {
     return a.K % 128 == 0 && aligned(a.xq, 16) && aligned(a.wq, 16) && a.ldx % 16 == 0 && a.ldw % 16 == 0 &&
@@ -682,7 +737,7 @@ extern "C" int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T,
     if (M == 0 || H == 0) return MX_OK;
     GroupedArgs a = base_args(xq, xs, ldx, ldxs, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
     a.hq = hq, a.ldhq = ldhq, a.hs = hs, a.ldhs = ldhs, a.pre = pre, a.ldpre = ldpre;
-    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 16) || ldpre % 8 || H % 8)))
+    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 8) || ldpre % 4)))
         return MX_EUNSUPPORTED;
     return launch_grouped_dt<MODE_GEMM1>(act_dtype, a, (hipStream_t)stream);
 }
@@ -725,6 +780,34 @@ extern "C" int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int6
         ldpre % 8 || H % 8 || !aligned(dpq, 8) || lddpq % 8)
         return MX_EUNSUPPORTED;
     return launch_grouped_dt<MODE_DGRAD2>(act_dtype, a, (hipStream_t)stream);
+}
+
+extern "C" int mx_experts_combine(const void *y, int64_t ldy, const int32_t *order, const int32_t *offsets, int64_t E,
+                                  const void *gate, int gate_dtype, int32_t *inv, int64_t T, int64_t top_k, void *out,
+                                  int dtype, int64_t ldo, int64_t M, int64_t N, void *stream) {
+    if (E <= 0 || E >= (1 << 20) || T < 0 || top_k <= 0 || top_k > 0x7FFF || M < 0 || N < 0 || M >= 0x7FFFFFFF ||
+        T * top_k >= 0x7FFFFFFF || ldy < N || ldo < N || !order || !offsets || !inv)
+        return MX_EINVAL;
+    if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EINVAL;
+    if (gate && gate_dtype != MX_FP32 && gate_dtype != dtype) return MX_EINVAL;
+    if (T == 0 || N == 0) return MX_OK;
+    if (N % 8 || !aligned(y, 16) || !aligned(out, 16) || ldy % 8 || ldo % 8) return MX_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t pairs = T * top_k;
+    fill_i32_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>(inv, pairs, -1);
+    if (M) invert_order_kernel<<<dim3((unsigned)((M + 255) / 256)), dim3(256), 0, st>>>(order, offsets, (int)E, M, pairs, inv);
+    const int n8 = (int)(N / 8);
+    const int64_t blocks = (T * n8 + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    if (dtype == MX_BF16)
+        combine_kernel<MX_BF16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const uint16_t *)y, ldy, inv, gate,
+                                                                             gate_dtype == MX_FP32, (int)top_k,
+                                                                             (uint16_t *)out, ldo, T, n8);
+    else
+        combine_kernel<MX_FP16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>((const uint16_t *)y, ldy, inv, gate,
+                                                                             gate_dtype == MX_FP32, (int)top_k,
+                                                                             (uint16_t *)out, ldo, T, n8);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
 template <int CDT>

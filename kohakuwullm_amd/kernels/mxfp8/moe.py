@@ -97,6 +97,40 @@ def launch_scatter_gemm(aq, a_s, wq, ws, out, token_of, order, gate, offsets, in
     )
 
 
+def combine_sorted_rows(y, order, offsets, num_experts, gate, tokens: int, top_k: int) -> torch.Tensor:
+    """``out[t] = sum_k gate[t*top_k+k] * y[position of pair t*top_k+k]``: the scatter-add as a gather.
+
+    ``order`` must be the pair index ``token * top_k + slot`` (what ``expert_sort`` produces).
+    Deterministic; every row of the result is written.
+    """
+    m, n = y.shape
+    out = torch.empty(tokens, n, device=y.device, dtype=y.dtype)
+    inv = torch.empty(tokens * top_k, device=y.device, dtype=torch.int32)
+    _lib.invoke(
+        "mx_experts_combine", y.element_size() * n * (tokens * top_k + tokens), y,
+        y.data_ptr(), y.stride(0), order.data_ptr(), offsets.data_ptr(), num_experts,
+        0 if gate is None else gate.data_ptr(), 0 if gate is None else _lib.MX_DTYPE[gate.dtype], inv.data_ptr(),
+        tokens, top_k, out.data_ptr(), _lib.MX_DTYPE[out.dtype], out.stride(0), m, n,
+    )
+    return out
+
+
+def _routed_product(aq, a_s, wq, ws, token_of, order, gate, offsets, tokens: int, top_k: int, dtype) -> torch.Tensor:
+    """``out[token] += scale * (a[m] . w[e(m)]^T)`` over the sorted rows.
+
+    When ``order`` is a pair index (``top_k`` > 0) the rows are written once by the grouped GEMM
+    and gathered per token; otherwise the scatter GEMM adds them into a zeroed output with
+    16-bit atomics, as the reference does.
+    """
+    n = wq.shape[1]
+    if top_k > 0 and n % 8 == 0:
+        y = grouped_mxfp8_gemm(aq, a_s, wq, ws, offsets, out_dtype=dtype, rows=token_of.numel())
+        return combine_sorted_rows(y, order, offsets, wq.shape[0], gate, tokens, top_k)
+    out = torch.zeros(tokens, n, device=aq.device, dtype=dtype)
+    launch_scatter_gemm(aq, a_s, wq, ws, out, token_of, order if gate is not None else None, gate, offsets)
+    return out
+
+
 def launch_gemm2_dgrad(dq, ds, token_of, order, gate, wq, ws, hq, hs, pre, dpre, dpq, dps, dgate, offsets) -> None:
     m = token_of.numel()
     hidden, dim = wq.shape[1], wq.shape[2]
@@ -123,19 +157,20 @@ class _MXFP8Experts(torch.autograd.Function):
         hs = torch.empty(m, hidden // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
         pre = torch.empty(m, 2 * hidden, device=x.device, dtype=x.dtype) if needs_grad else None
         launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hidden, dim, x.dtype)
-        out = torch.zeros(rows, dim, device=x.device, dtype=x.dtype)
-        launch_scatter_gemm(hq, hs, *packed.out_fwd, out, token_of, order, gate, offsets)
+        # pairs per token when `order` is the pair index token * top_k + slot; 0 = unknown layout
+        top_k = gate.numel() // rows if rows and gate.numel() % rows == 0 else 0
+        out = _routed_product(hq, hs, *packed.out_fwd, token_of, order, gate, offsets, rows, top_k, x.dtype)
         if needs_grad:
             ctx.save_for_backward(x, hq, hs, pre, gate, token_of, order, offsets)
             ctx.packed = packed
-            ctx.shapes = (hidden, dim, m, rows)
+            ctx.shapes = (hidden, dim, m, rows, top_k)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         x, hq, hs, pre, gate, token_of, order, offsets = ctx.saved_tensors
         packed = ctx.packed
-        hidden, dim, m, rows = ctx.shapes
+        hidden, dim, m, rows, top_k = ctx.shapes
         dev = dout.device
         dout = dout.contiguous()
         dq, ds = quantize_mx(dout)
@@ -145,8 +180,7 @@ class _MXFP8Experts(torch.autograd.Function):
         # fp32 and zeroed: this reduction crosses workgroups through an atomic
         dgate = torch.zeros(gate.numel(), device=dev, dtype=torch.float32)
         launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets)
-        dx = torch.zeros(rows, dim, device=dev, dtype=dout.dtype)
-        launch_scatter_gemm(dpq, dps, *packed.in_dgrad, dx, token_of, None, None, offsets)
+        dx = _routed_product(dpq, dps, *packed.in_dgrad, token_of, order, None, offsets, rows, top_k, dout.dtype)
 
         dw_in = dw_out = None
         if ctx.needs_input_grad[2]:
