@@ -185,6 +185,11 @@ def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
     }
 
 
+# Bytes the GEMM launches of one step move between the L2s and the fabric, per launch, from the
+# FETCH_SIZE and WRITE_SIZE counter runs summarised under profiles/ (each scaled by what the
+# counter reads for a device copy of known size): 3090 MiB over 4 launches.
+GEMM_TRAFFIC_PER_LAUNCH = {"ffn": 772 * 2**20}
+
 GEMM_ENTRIES = ("mx_gemm_nt", "mx_gemm_nt_batch", "mx_grouped_gemm_nt", "mx_experts_gemm1", "mx_experts_scatter_gemm",
                 "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt")
 
@@ -286,6 +291,9 @@ def main() -> None:
                     help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed region, run one device copy of 256 MiB: a kernel of known traffic "
+                         "against which a counter run (FETCH_SIZE / WRITE_SIZE) is scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this path is built and run on a single GPU (--gpus 1)")
@@ -316,6 +324,13 @@ def main() -> None:
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     tflops = gflop / ms_per_step
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # Instrumented pass: the same steps with events around every kernel launch.
     _lib.TIMER = []
@@ -364,7 +379,7 @@ def main() -> None:
             "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(gemm_tflops / MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_PER_LAUNCH.get(args.workload),
             "launches": len(gemm),
             "avg_launch_us": round(gemm_ms / len(gemm) * 1e3, 2),
             "gflop_per_launch": round(gemm_flops / len(gemm) / 1e9, 2),
