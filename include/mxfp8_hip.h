@@ -122,6 +122,19 @@ int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, in
                                 uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
 
 /*
+ * Scale layout interop.  The reference's cuBLAS route keeps UE8M0 scales in the flat
+ * SWIZZLE_32_4_4 layout: 128-row x 4-column tiles of 512 bytes, row-tile major, scale
+ * (r, c) of a tile at (r % 32) * 16 + (r / 32) * 4 + c, zero padded to whole tiles
+ * (ceil(rows/128)*128 * ceil(cols/4)*4 bytes).  The MI355X kernels read the natural
+ * (rows, cols) layout; these two convert either way so tensors produced for, or by, the
+ * reference's quantize_mx_vendor / mxfp8_mm_swizzled can be exchanged.
+ * Replaces swizzle_mx_scales (src/kohakuwullm/kernels/mxfp8/interop.py:24-41) and the
+ * swizzled store of _quantize_mx_vendor_kernel (quantize.py:175-180).
+ */
+int mx_swizzle_scales(const uint8_t *s, int64_t rows, int64_t cols, int64_t lds, uint8_t *swizzled, void *stream);
+int mx_unswizzle_scales(const uint8_t *swizzled, int64_t rows, int64_t cols, uint8_t *s, int64_t lds, void *stream);
+
+/*
  * C (M,N) = deq(A) deq(B)^T, fp32 accumulate, cast to c_dtype (round to nearest
  * even).  A: codes (M,K) pitch lda + scales (M,K/32) pitch ldas; B: codes (N,K)
  * pitch ldb + scales (N,K/32) pitch ldbs; both K-minor.  K % 32 == 0.

@@ -692,3 +692,62 @@ extern "C" int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, i
     MX_LAUNCH_CHECK();
     return MX_OK;
 }
+
+// ---- cuBLAS SWIZZLE_32_4_4 scale layout (interop) -------------------------------------------------
+// 128-row x 4-column tiles of 512 bytes, row-tile major; inside a tile scale (r, c) sits at
+// (r % 32) * 16 + (r / 32) * 4 + c; zero padded to whole tiles.  One thread moves the 4 bytes
+// of one row of one tile.  (src/kohakuwullm/kernels/mxfp8/interop.py:24-41, quantize.py:175-180.)
+namespace mx {
+template <bool TO_SWIZZLED>
+__global__ __launch_bounds__(256) void swizzle_scales_kernel(uint8_t *__restrict__ natural, int64_t lds,
+                                                             uint8_t *__restrict__ swizzled, int64_t rows, int64_t cols,
+                                                             int64_t col_tiles, int64_t total) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one dword of the swizzled buffer
+    if (idx >= total) return;
+    const int64_t tile = idx >> 7;
+    const int in = (int)(idx & 127);        // (r % 32) * 4 + r / 32
+    const int rr = (in >> 2) + 32 * (in & 3);
+    const int64_t r = (tile / col_tiles) * 128 + rr;
+    const int64_t c0 = (tile % col_tiles) * 4;
+    if (TO_SWIZZLED) {
+        uint32_t w = 0;
+        if (r < rows)
+            for (int c = 0; c < 4; c++)
+                if (c0 + c < cols) w |= (uint32_t)natural[r * lds + c0 + c] << (8 * c);
+        ((uint32_t *)swizzled)[idx] = w;
+    } else if (r < rows) {
+        const uint32_t w = ((const uint32_t *)swizzled)[idx];
+        for (int c = 0; c < 4; c++)
+            if (c0 + c < cols) natural[r * lds + c0 + c] = (uint8_t)(w >> (8 * c));
+    }
+}
+}  // namespace mx
+
+static int swizzle_launch(bool to_swizzled, uint8_t *natural, int64_t lds, uint8_t *swizzled, int64_t rows, int64_t cols,
+                          void *stream) {
+    if (rows < 0 || cols < 0 || lds < cols) return MX_EINVAL;
+    if (((uintptr_t)swizzled & 3) != 0) return MX_EINVAL;
+    const int64_t row_tiles = (rows + 127) / 128, col_tiles = (cols + 3) / 4;
+    const int64_t total = row_tiles * col_tiles * 128;
+    if (total == 0) return MX_OK;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (to_swizzled)
+        mx::swizzle_scales_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(natural, lds, swizzled, rows, cols,
+                                                                                    col_tiles, total);
+    else
+        mx::swizzle_scales_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(natural, lds, swizzled, rows, cols,
+                                                                                     col_tiles, total);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+extern "C" int mx_swizzle_scales(const uint8_t *s, int64_t rows, int64_t cols, int64_t lds, uint8_t *swizzled,
+                                 void *stream) {
+    return swizzle_launch(true, (uint8_t *)s, lds, swizzled, rows, cols, stream);
+}
+
+extern "C" int mx_unswizzle_scales(const uint8_t *swizzled, int64_t rows, int64_t cols, uint8_t *s, int64_t lds,
+                                   void *stream) {
+    return swizzle_launch(false, s, lds, (uint8_t *)swizzled, rows, cols, stream);
+}

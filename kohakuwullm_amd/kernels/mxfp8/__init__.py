@@ -16,6 +16,15 @@ from kohakuwullm_amd.kernels.mxfp8.quantize import (
     quantize_mx_dual,
 )
 
+
+
+def quantize_mx_vendor(x):
+    """``quantize_mx`` with swizzled e8m0 scales (``quantize.py:140-215`` of the reference); see :mod:`interop`."""
+    from kohakuwullm_amd.kernels.mxfp8.interop import quantize_mx_vendor as impl
+
+    return impl(x)
+
+
 __all__ = [
     "BLOCK_SCALE",
     "E4M3_MAX",
@@ -25,4 +34,5 @@ __all__ = [
     "quantize_mx",
     "quantize_mx_cols",
     "quantize_mx_dual",
+    "quantize_mx_vendor",
 ]
