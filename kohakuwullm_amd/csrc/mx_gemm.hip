@@ -293,9 +293,10 @@ static int num_cus() {
     return n;
 }
 
-// Scratch of the even K split: two fp32 tile slots per workgroup, kept per (device, stream)
-// for the life of the process so launches on different streams never share it.
-static float *split_scratch(hipStream_t st, int cus, size_t tile_floats) {
+// Scratch of the K splits (dense and expert WGRAD): two fp32 tile slots per workgroup, kept per
+// (device, stream) for the life of the process so launches on different streams never share it.
+namespace mx {
+float *split_scratch(hipStream_t st, int cus, size_t tile_floats) {
     static std::mutex lock;
     static std::map<std::pair<int, hipStream_t>, float *> table;
     int dev = 0;
@@ -317,6 +318,7 @@ static float *split_scratch(hipStream_t st, int cus, size_t tile_floats) {
     table[key] = slots;  // a failed allocation is remembered: the library keeps working on whole tiles
     return slots;
 }
+}  // namespace mx
 
 // MX_GEMM_SPLIT=0 in the environment keeps every tile whole (for A/B timing and debugging).
 static bool split_mode() {

@@ -21,6 +21,8 @@
 
 namespace mx {
 
+float *split_scratch(hipStream_t st, int cus, size_t tile_floats);  // mx_gemm.hip
+
 enum { MODE_PLAIN = 0, MODE_GEMM1 = 1, MODE_SCATTER = 2, MODE_DGRAD2 = 3 };
 
 struct GroupedArgs {
@@ -518,54 +520,120 @@ struct WgradArgs {
     const int32_t *offsets;
     int E, N, Kout, KB;  // KB: scale bytes per row of the padded space
     int tiles_m, tiles_n, c_vec;
+    // K split for few, long tiles (a handful of busy experts): `slots` fp32 tile slots; every
+    // workgroup derives the same number of K slices per tile from the offsets (wgrad_slices),
+    // slice s of the j-th tile of a non-empty expert leaves its partial sum in slot j * slices + s,
+    // and wgrad_reduce_kernel adds the slices in order.  slots == 0: whole tiles only.
+    float *ws;
+    int slots;
 };
+
+// Number of K slices per tile: as many as fill the GPU about twice over, at most 8, and 1 when
+// the tiles of the non-empty experts already fill three quarters of it.  Also counts the
+// non-empty experts.
+__device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, int &live) {
+    live = 0;
+    for (int e = 0; e < p.E; e++) live += p.offsets[e + 1] > p.offsets[e] ? 1 : 0;
+    const int tiles = live * p.tiles_m * p.tiles_n;
+    if (!p.slots || tiles == 0 || tiles * 4 >= workgroups * 3) return 1;
+    int s = 2 * workgroups / tiles;
+    s = s < p.slots / tiles ? s : p.slots / tiles;
+    return s < 1 ? 1 : (s > 8 ? 8 : s);
+}
 
 template <typename S, int CDT>
 struct WgradProblem {
     struct Tile {
         int m0, n0, kt0, kt1, expert;
+        int slot;  // fp32 scratch slot of this K slice, or -1 for a whole tile
     };
     const WgradArgs p;
-    int next_id, kb_end, scan_e, scan_tiles;
+    // Units are dealt round-robin over the workgroups: first the (tile, K slice) units of the
+    // non-empty experts, compactly numbered so they spread evenly wherever those experts sit
+    // among the E, then the tiles of the empty experts, which are only zero-filled.
+    int next_unit, next_dead, kb_end;
+    int live, slices;
+    // incremental scans: expert scan_e is the scan_live-th non-empty one and its first K stage
+    // is scan_tiles; expert dead_e is the dead_seen-th empty one
+    int scan_e, scan_tiles, scan_live, dead_e, dead_seen;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
-    __device__ WgradProblem(const WgradArgs &a) : p(a), next_id(blockIdx.x), kb_end(a.KB), scan_e(0), scan_tiles(0) {}
+    __device__ WgradProblem(const WgradArgs &a)
+        : p(a), next_unit(blockIdx.x), next_dead(blockIdx.x), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0),
+          dead_e(0), dead_seen(0) {
+        slices = wgrad_slices(p, (int)gridDim.x, live);
+    }
 
-    __device__ __forceinline__ void zero_tile(const Tile &t) const {
+    __device__ __forceinline__ void zero_tile(int expert, int m0, int n0) const {
         // an expert without rows: its dW tile is zeros
         const int esz = CDT == MX_FP32 ? 4 : 2;
+        char *base = (char *)p.dw + (int64_t)expert * p.stride_dwe * esz;
+        if (p.c_vec && m0 + S::BM <= p.N && n0 + S::BN <= p.Kout) {
+            constexpr int PER_ROW = S::BN * esz / 16;
+            for (int idx = threadIdx.x; idx < S::BM * PER_ROW; idx += S::NTHR) {
+                const int m = m0 + idx / PER_ROW, c = idx % PER_ROW;
+                *(v4i *)(base + ((int64_t)m * p.lddw + n0) * esz + c * 16) = v4i{0, 0, 0, 0};
+            }
+            return;
+        }
         for (int idx = threadIdx.x; idx < S::BM * S::BN; idx += S::NTHR) {
-            const int m = t.m0 + idx / S::BN, n = t.n0 + idx % S::BN;
+            const int m = m0 + idx / S::BN, n = n0 + idx % S::BN;
             if (m < p.N && n < p.Kout) {
-                char *dst = (char *)p.dw + ((int64_t)t.expert * p.stride_dwe + (int64_t)m * p.lddw + n) * esz;
+                char *dst = base + ((int64_t)m * p.lddw + n) * esz;
                 if (esz == 4) *(float *)dst = 0.0f;
                 else *(uint16_t *)dst = 0;
             }
         }
     }
 
+    __device__ __forceinline__ void zero_slot(int slot) const {
+        v4f *dst = (v4f *)p.ws + (int64_t)slot * (S::BM * S::BN / 4);
+        for (int idx = threadIdx.x; idx < S::BM * S::BN / 4; idx += S::NTHR) dst[idx] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+
     __device__ __forceinline__ bool next(Tile &t) {
         const int per_e = p.tiles_m * p.tiles_n;
-        while (next_id < per_e * p.E) {
-            const int id = next_id;
-            next_id += gridDim.x;
-            const int e = id / per_e;
-            const int rem = id - e * per_e;
-            // tiles of experts before e (ids, hence e, only grow for one workgroup)
-            while (scan_e < e) {
-                scan_tiles += (p.offsets[scan_e + 1] - p.offsets[scan_e] + 127) / 128;
+        const int per_live = per_e * slices;
+        while (next_unit < live * per_live) {
+            const int unit = next_unit;
+            next_unit += gridDim.x;
+            const int j = unit / per_live, r = unit - j * per_live;
+            const int slice = r / per_e, rem = r - slice * per_e;  // slice-major: neighbours share operand panels
+            // advance to the j-th non-empty expert (units, hence j, only grow for one workgroup)
+            while (true) {
+                const int rows = p.offsets[scan_e + 1] - p.offsets[scan_e];
+                if (rows > 0 && scan_live == j) break;
+                scan_tiles += (rows + 127) / 128;
+                scan_live += rows > 0 ? 1 : 0;
                 scan_e++;
             }
-            t.expert = e;
+            t.expert = scan_e;
             t.m0 = (rem / p.tiles_n) * S::BM;
             t.n0 = (rem % p.tiles_n) * S::BN;
-            t.kt0 = scan_tiles;
-            t.kt1 = scan_tiles + (p.offsets[e + 1] - p.offsets[e] + 127) / 128;
-            if (t.kt0 == t.kt1) {
-                zero_tile(t);
+            const int len = (p.offsets[scan_e + 1] - p.offsets[scan_e] + 127) / 128;
+            const int per = (len + slices - 1) / slices;
+            const int lo = slice * per < len ? slice * per : len;
+            const int hi = lo + per < len ? lo + per : len;
+            t.kt0 = scan_tiles + lo;
+            t.kt1 = scan_tiles + hi;
+            t.slot = slices > 1 ? (j * per_e + rem) * slices + slice : -1;
+            if (lo == hi) {
+                zero_slot(t.slot);  // only a slice can be empty: a whole tile of a non-empty expert has K stages
                 continue;
             }
             return true;
+        }
+        const int dead_tiles = (p.E - live) * per_e;
+        while (next_dead < dead_tiles) {
+            const int d = next_dead / per_e, rem = next_dead - d * per_e;
+            next_dead += gridDim.x;
+            while (true) {
+                const bool empty = p.offsets[dead_e + 1] <= p.offsets[dead_e];
+                if (empty && dead_seen == d) break;
+                dead_seen += empty ? 1 : 0;
+                dead_e++;
+            }
+            zero_tile(dead_e, (rem / p.tiles_n) * S::BM, (rem % p.tiles_n) * S::BN);
         }
         return false;
     }
@@ -604,6 +672,14 @@ struct WgradProblem {
     }
 
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+        if (t.slot >= 0) {  // one K slice: fp32 partial, laid out [sub-tile][thread]
+            v4f *dst = (v4f *)p.ws + (int64_t)t.slot * (S::BM * S::BN / 4);
+#pragma unroll
+            for (int i = 0; i < S::MT; i++)
+#pragma unroll
+                for (int j = 0; j < S::NT; j++) dst[(i * S::NT + j) * S::NTHR + L.tid] = acc[i][j];
+            return -1;
+        }
         const bool interior = t.m0 + S::BM <= p.N && t.n0 + S::BN <= p.Kout && p.c_vec;
         const int64_t base = (int64_t)t.expert * p.stride_dwe;
         const int n = t.n0 + L.wn * S::WTN + 8 * L.r16;
@@ -628,6 +704,50 @@ __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     WgradProblem<S, CDT> prob(args);
     persistent_gemm<S, false>(prob, smem);
+}
+
+// Adds the K slices of every tile of every non-empty expert, in slice order, and stores dW.
+// One block per (tile of a non-empty expert, i), numbered compactly as in the GEMM; the grid is
+// sized for E experts, so blocks past the non-empty ones, and all blocks when the GEMM kept its
+// tiles whole, have nothing to do.
+template <typename S, int CDT>
+__global__ __launch_bounds__(S::NTHR) void wgrad_reduce_kernel(WgradArgs p, int workgroups) {
+    int live;
+    const int slices = wgrad_slices(p, workgroups, live);
+    if (slices == 1) return;
+    const int per_e = p.tiles_m * p.tiles_n;
+    const int id = blockIdx.x / S::MT, i = blockIdx.x % S::MT;
+    const int j = id / per_e, rem = id - j * per_e;
+    if (j >= live) return;
+    int e = 0;
+    for (int seen = 0;; e++) {
+        if (p.offsets[e + 1] > p.offsets[e]) {
+            if (seen == j) break;
+            seen++;
+        }
+    }
+    const int tid = threadIdx.x;
+    v4f sum[S::NT];
+#pragma unroll
+    for (int jj = 0; jj < S::NT; jj++) sum[jj] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int sl = 0; sl < slices; sl++) {
+        const v4f *src = (const v4f *)p.ws + (int64_t)((j * per_e + rem) * slices + sl) * (S::BM * S::BN / 4);
+#pragma unroll
+        for (int jj = 0; jj < S::NT; jj++) sum[jj] += src[(i * S::NT + jj) * S::NTHR + tid];
+    }
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave / S::WGN, wn = wave % S::WGN;
+    const int n = (rem % p.tiles_n) * S::BN + wn * S::WTN + 8 * (lane & 15);
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int m = (rem / p.tiles_n) * S::BM + wm * S::WTM + 16 * i + 4 * (lane >> 4) + v;
+        if (m < p.N && n < p.Kout) {
+            const v4f lo = {sum[0][v], sum[1][v], sum[2][v], sum[3][v]};
+            const v4f hi = {sum[4][v], sum[5][v], sum[6][v], sum[7][v]};
+            store8<CDT>(p.dw, (int64_t)e * p.stride_dwe + (int64_t)m * p.lddw + n, lo, hi, p.Kout - n < 8 ? p.Kout - n : 8,
+                        p.c_vec != 0);
+        }
+    }
 }
 
 }  // namespace mx
@@ -820,11 +940,16 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
     const int64_t work = (int64_t)a.tiles_m * a.tiles_n * a.E;
     if (work >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
     const int cus = num_cus();
-    dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
+    // With more tile ids than workgroups the K split can still pay: the ids of experts without
+    // rows are empty, and how many those are is only known on the device.
+    a.ws = work < (1 << 27) ? mx::split_scratch(st, cus, (size_t)S::BM * S::BN) : nullptr;
+    a.slots = a.ws ? 2 * cus : 0;
+    dim3 grid((unsigned)(work * (a.slots ? 8 : 1) < cus ? work * (a.slots ? 8 : 1) : cus)), block(S::NTHR);
     auto kern = grouped_wgrad_kernel<S, CDT>;
     if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
         return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    if (a.slots) wgrad_reduce_kernel<S, CDT><<<dim3((unsigned)(work * S::MT)), block, 0, st>>>(a, (int)grid.x);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
