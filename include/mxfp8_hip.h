@@ -192,12 +192,19 @@ int mx_grouped_gemm_nt(const uint8_t *xq, const uint8_t *xs, int64_t a_rows, int
  * Expert GEMM1 with its epilogue: rows gathered by token_of, both halves of x . w_in^T
  * (w_in (E,2H,K), gate rows first), accumulators rounded to act_dtype, optional store of
  * pre (M,2H), h = gate * sigmoid(gate) * value quantized per 32 of H into hq (M,H), hs (M,H/32).
+ * token_of == NULL gathers nothing (row m is x row m).  With htq/hts != NULL the same h is
+ * also quantized along the tokens, into the padded layout of mx_quantize_cols_grouped
+ * ((H,Mpad), (H,Mpad/32); with E == 1 and M % 128 == 0 that is plain (H,M)): the operand of
+ * GEMM2's WGRAD, bit-identical to mx_quantize_cols_grouped(pre, source = SwiGLU).
+ * With E == 1 this is the dense SwiGLU block's first projection with the activation and both
+ * casts in the epilogue (GLUMLP.forward, src/kohakuwullm/models/components/mlp.py:68-73).
  * Replaces _experts_gemm1 / launch_gemm1 (src/kohakuwullm/kernels/mxfp8/experts.py:25-135,225-275).
  */
 int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T, int64_t ldx, int64_t ldxs,
                      const int32_t *token_of, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
                      int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
                      uint8_t *hq, int64_t ldhq, uint8_t *hs, int64_t ldhs, void *pre, int64_t ldpre,
+                     uint8_t *htq, int64_t ldhtq, uint8_t *hts, int64_t ldhts,
                      int act_dtype, int64_t M, int64_t H, int64_t K, void *stream);
 
 /*

@@ -38,7 +38,7 @@ SIGNATURES = {
         _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p]),
     "mx_experts_gemm1": (
         _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64,
-              _ci, _i64, _i64, _i64, _p]),
+              _p, _i64, _p, _i64, _ci, _i64, _i64, _i64, _p]),
     "mx_experts_scatter_gemm": (
         _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _p, _p, _ci, _p, _ci, _i64,
               _i64, _i64, _i64, _p]),

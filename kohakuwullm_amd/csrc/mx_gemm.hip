@@ -151,7 +151,7 @@ struct DenseProblem {
             for (int j = 0; j < S::NT; j++) mine[(i * S::NT + j) * S::NTHR + L.tid] = acc[i][j];
     }
 
-    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
         if (t.sk >= 0) {
             write_piece(t, L, acc);
             return -1;

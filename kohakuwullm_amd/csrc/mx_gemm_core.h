@@ -359,13 +359,21 @@ __device__ __forceinline__ void wait_vm_allow_c() {
     __builtin_amdgcn_s_waitcnt(((N & 15) | (7 << 4) | ((N >> 4) << 14)));
 }
 
+// The two halves (A part, B part: DATA_A and DATA_B bytes) of the LDS stage buffer the tile's
+// last K stage was read from.  An epilogue may use them as scratch once every wave has left
+// the main loop (a workgroup barrier of its own first); the buffer is not written again before
+// the barrier that follows the epilogue.
+struct LdsScratch {
+    uint8_t *a, *b;
+};
+
 // The persistent tile loop.  `P` (the problem policy) provides
 //   bool P::next(Tile &t)                   advance to this workgroup's next tile (false = done);
 //                                           tiles with an empty K range are finished inside next()
 //   void P::context(const Tile &, const Lane &, IssueCtx<S> &)
 //   const uint8_t *P::line(const Tile &, int operand_row)   address of K byte 0 of row
 //                                           operand_row of the [A rows; B rows] list (for L2 touches)
-//   int  P::epilogue(const Tile &, const Lane &, v4f (&acc)[MT][NT])   returns how many stores each
+//   int  P::epilogue(const Tile &, const Lane &, v4f (&acc)[MT][NT], const LdsScratch &)   returns how many stores each
 //                                           lane issued if that number is the same compile-time
 //                                           constant P::NST for the whole wave, else -1
 //   int  P::kb_end                          scale bytes per row (bound for predicated fetches)
@@ -496,7 +504,8 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         // conversions run under that latency, and when every lane issued the same known number
         // of stores the wait lets exactly those (and the L2 touch before them) stay in flight,
         // so the stores drain under the next tile's first stage.
-        const int stores = prob.epilogue(cur, L, acc);
+        const int lastbuf = (gstage - 1) & 1;
+        const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B});
         if (has_next) {
             if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
             if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);

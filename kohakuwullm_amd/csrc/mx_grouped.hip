@@ -45,6 +45,8 @@ struct GroupedArgs {
     int gate_f32;
     uint8_t *hq, *hs;  // GEMM1 out / DGRAD2 in: (M,H), (M,H/32)
     int64_t ldhq, ldhs;
+    uint8_t *htq, *hts;  // GEMM1 out (optional): h quantized along the tokens, (H,Mpad), (H,Mpad/32)
+    int64_t ldhtq, ldhts;
     void *pre;  // GEMM1 out (optional) / DGRAD2 in: (M,2H) 16-bit
     int64_t ldpre;
     void *dpre;  // DGRAD2 out: (M,2H) 16-bit
@@ -130,12 +132,14 @@ template <typename S, int MODE, int CDT>
 struct GroupedProblem {
     struct Tile {
         int n0, row0, end, expert, kt0, kt1;
+        int ppos;  // position of row0 in the padded token axis (each expert padded to 128-row tiles)
     };
     const GroupedArgs p;  // a copy: fields live in scalar registers
     int next_id;
     int kb_end;
-    // incremental tile_owner: experts [0, scan_e) own row tiles [0, scan_tiles)
-    int scan_e, scan_tiles;
+    // incremental tile_owner: experts [0, scan_e) own row tiles [0, scan_tiles) and the first
+    // scan_pad 128-row tiles of the padded token axis
+    int scan_e, scan_tiles, scan_pad;
 
     // Accumulator layout (GemmShape LANES_N): lane (r16, g) holds, for sub-tile (i, j) and
     // register v, row 16 i + 4 g + v of the wave's 64 rows and column 8 r16 + j of its 128.
@@ -147,7 +151,7 @@ struct GroupedProblem {
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
     __device__ GroupedProblem(const GroupedArgs &a)
-        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0) {}
+        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0), scan_pad(0) {}
 
     __device__ __forceinline__ bool next(Tile &t) {
         const int total = p.tiles_n * p.tbound;
@@ -163,8 +167,9 @@ struct GroupedProblem {
             if (rt < scan_tiles) {  // ids are monotonic per workgroup except across the XCD remap edge
                 scan_e = 0;
                 scan_tiles = 0;
+                scan_pad = 0;
             }
-            int e = scan_e, before = scan_tiles, start = 0, end = 0;
+            int e = scan_e, before = scan_tiles, pad = scan_pad, start = 0, end = 0;
             bool found = false;
             while (e < p.E) {
                 start = p.offsets[e];
@@ -175,14 +180,17 @@ struct GroupedProblem {
                     break;
                 }
                 before += tiles;
+                pad += (end - start + 127) / 128;
                 e++;
             }
             scan_e = e;
             scan_tiles = before;
+            scan_pad = pad;
             if (!found) continue;  // past the last real row tile
             t.expert = e;
             t.row0 = start + (rt - before) * S::BM;
             t.end = end;
+            t.ppos = pad * 128 + (rt - before) * S::BM;
             t.n0 = tn * N_PER_TILE;
             t.kt0 = 0;
             t.kt1 = p.K >> 7;
@@ -239,11 +247,12 @@ struct GroupedProblem {
         return p.wq + (int64_t)t.expert * p.stride_we + (int64_t)b_src_row(t, r - S::BM) * p.ldw;
     }
 
-    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
-        if (MODE == MODE_PLAIN) return epilogue_plain(t, L, acc);
-        if (MODE == MODE_GEMM1) return epilogue_gemm1(t, L, acc);
-        if (MODE == MODE_SCATTER) return epilogue_scatter(t, L, acc);
-        return epilogue_dgrad2(t, L, acc);
+    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT],
+                                            const LdsScratch &lds) const {
+        if constexpr (MODE == MODE_PLAIN) return epilogue_plain(t, L, acc);
+        else if constexpr (MODE == MODE_GEMM1) return epilogue_gemm1(t, L, acc, lds);
+        else if constexpr (MODE == MODE_SCATTER) return epilogue_scatter(t, L, acc);
+        else return epilogue_dgrad2(t, L, acc);
     }
 
     // sorted row of (i, v) for this lane
@@ -271,42 +280,105 @@ struct GroupedProblem {
     }
 
     // ---- GEMM1: sub-tiles 0-3 are gate, 4-7 value of the lane's 4 hidden units
-    __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+    // Outputs: pre (rounded accumulators), h quantized along the hidden axis (hq, hs) for GEMM2,
+    // and, when htq is given, h quantized along the tokens for GEMM2's WGRAD.  The token-axis
+    // blocks are the 32-row groups (i, i+1) x g x v of a wave; their codes are transposed through
+    // the LDS stage buffer the main loop has just left, so they reach memory as 256-byte runs.
+    // (The epilogue is bound by its vector ALU work -- rounding, sigmoid, two quantizers per
+    // value -- not by its stores: staging the row-direction outputs through LDS for wider
+    // stores was measured and did not pay.)
+    __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT],
+                                                  const LdsScratch &lds) const {
+        static_assert(S::MT % 2 == 0 && N_PER_TILE * S::BM <= S::DATA_A, "token-axis staging: one A half holds the tile");
         const int hblock = t.n0 + L.wn * (S::WTN / 2) + 32 * (L.r16 >> 3);  // the 32 hidden units of 8 lanes
         const int h = t.n0 + L.wn * (S::WTN / 2) + 4 * L.r16;
+        const bool tok = p.htq != nullptr;
+        if (tok) __syncthreads();  // every wave is out of the main loop: the stage buffer is free
 #pragma unroll
-        for (int i = 0; i < S::MT; i++) {
+        for (int blk = 0; blk < S::MT / 2; blk++) {
+            float a[2][4][4];  // [i in block][v][hidden unit]
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int m = row_of(t, L, i, v);
-                const bool ok = m < t.end && hblock < p.N;  // H % 32 == 0: a block is in or out
-                float gv[4], vv[4];
-                uint32_t gp[2], vp[2];
+            for (int ii = 0; ii < 2; ii++) {
+                const int i = 2 * blk + ii;
 #pragma unroll
-                for (int e = 0; e < 4; e++) gv[e] = acc[i][e][v], vv[e] = acc[i][4 + e][v];
-                // h is rounded to the storage dtype before the activation, so the backward
-                // differentiates the function the forward evaluated (experts.py:116-119)
+                for (int v = 0; v < 4; v++) {
+                    const int m = row_of(t, L, i, v);
+                    const bool row_ok = m < t.end;
+                    const bool ok = row_ok && hblock < p.N;  // H % 32 == 0: a block is in or out
+                    float gv[4], vv[4];
+                    uint32_t gp[2], vp[2];
 #pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    round_pair<CDT>(gv[2 * e], gv[2 * e + 1], gp[e]);
-                    round_pair<CDT>(vv[2 * e], vv[2 * e + 1], vp[e]);
-                }
-                if (ok && p.pre) {
-                    uint16_t *pp = (uint16_t *)p.pre + (int64_t)m * p.ldpre + h;
-                    *(v2i *)pp = v2i{(int)gp[0], (int)gp[1]};
-                    *(v2i *)(pp + p.N) = v2i{(int)vp[0], (int)vp[1]};
-                }
-                float a[4];
+                    for (int e = 0; e < 4; e++) gv[e] = acc[i][e][v], vv[e] = acc[i][4 + e][v];
+                    // h is rounded to the storage dtype before the activation, so the backward
+                    // differentiates the function the forward evaluated (experts.py:116-119)
 #pragma unroll
-                for (int e = 0; e < 4; e++) a[e] = gv[e] * sigmoid_f(gv[e]) * vv[e];
-                const float amax = oct_max(fmaxf(fmaxf(fabsf(a[0]), fabsf(a[1])), fmaxf(fabsf(a[2]), fabsf(a[3]))));
-                const uint32_t byte = scale_byte(amax);
-                const float inv = inv_scale(byte);
-                if (ok) {
-                    *(uint32_t *)(p.hq + (int64_t)m * p.ldhq + h) = pack4_e4m3(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv);
-                    if ((L.r16 & 7) == 0) p.hs[(int64_t)m * p.ldhs + (hblock >> 5)] = (uint8_t)byte;
+                    for (int e = 0; e < 2; e++) {
+                        round_pair<CDT>(gv[2 * e], gv[2 * e + 1], gp[e]);
+                        round_pair<CDT>(vv[2 * e], vv[2 * e + 1], vp[e]);
+                    }
+                    if (ok && p.pre) {
+                        uint16_t *pp = (uint16_t *)p.pre + (int64_t)m * p.ldpre + h;
+                        *(v2i *)pp = v2i{(int)gp[0], (int)gp[1]};
+                        *(v2i *)(pp + p.N) = v2i{(int)vp[0], (int)vp[1]};
+                    }
+                    float r[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = gv[e] * sigmoid_f(gv[e]) * vv[e];
+                    const float amax = oct_max(fmaxf(fmaxf(fabsf(r[0]), fabsf(r[1])), fmaxf(fabsf(r[2]), fabsf(r[3]))));
+                    const uint32_t byte = scale_byte(amax);
+                    const float inv = inv_scale(byte);
+                    if (ok) {
+                        *(uint32_t *)(p.hq + (int64_t)m * p.ldhq + h) = pack4_e4m3(r[0] * inv, r[1] * inv, r[2] * inv, r[3] * inv);
+                        if ((L.r16 & 7) == 0) p.hs[(int64_t)m * p.ldhs + (hblock >> 5)] = (uint8_t)byte;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) a[ii][v][e] = row_ok ? r[e] : 0.0f;  // rows past the expert are padding
                 }
             }
+            if (!tok) continue;
+            // token axis: the block's 32 rows are this lane's 8 values and the lanes 16, 32, 48 away
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float cm = 0.0f;
+#pragma unroll
+                for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) cm = fmaxf(cm, fabsf(a[ii][v][e]));
+                cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+                cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+                const uint32_t byte = scale_byte(cm);
+                const float inv = inv_scale(byte);
+                const int col = L.wn * (S::WTN / 2) + 4 * L.r16 + e;  // hidden unit inside the tile
+#pragma unroll
+                for (int ii = 0; ii < 2; ii++) {
+                    const int row = L.wm * S::WTM + 16 * (2 * blk + ii) + 4 * L.g;  // 4 consecutive rows: one dword
+                    const uint32_t w = pack4_e4m3(a[ii][0][e] * inv, a[ii][1][e] * inv, a[ii][2][e] * inv, a[ii][3][e] * inv);
+                    // column-major, 256 bytes per hidden unit, 16-byte chunks XOR-swizzled by the lane's r16
+                    *(uint32_t *)(lds.a + col * S::BM + ((((row >> 4) ^ (col >> 2)) & 15) << 4) + (row & 15)) = w;
+                }
+                if (L.g == 0) lds.b[col * (S::BM / 32) + L.wm * (S::WTM / 32) + blk] = (uint8_t)byte;
+            }
+        }
+        if (!tok) return -1;
+        __syncthreads();
+        // 16 consecutive lanes write the 256 bytes of one hidden unit's 256 tokens; a 128-row half
+        // that starts past the expert's rows belongs to the next expert's padding and is skipped
+        const int64_t pbase = t.ppos;
+#pragma unroll
+        for (int k = 0; k < N_PER_TILE * S::BM / 16 / S::NTHR; k++) {
+            const int q = L.tid + k * S::NTHR;
+            const int col = q >> 4, ch = q & 15;
+            const bool half_ok = t.row0 + (ch >> 3) * 128 < t.end;
+            if (t.n0 + col < p.N && half_ok) {
+                const v4i w = *(const v4i *)(lds.a + col * S::BM + (((ch ^ (col >> 2)) & 15) << 4));
+                *(v4i *)(p.htq + (int64_t)(t.n0 + col) * p.ldhtq + pbase + ch * 16) = w;
+            }
+        }
+        if (L.tid < N_PER_TILE && t.n0 + L.tid < p.N) {
+            const uint32_t *src = (const uint32_t *)(lds.b + L.tid * (S::BM / 32));
+            uint8_t *dst = p.hts + (int64_t)(t.n0 + L.tid) * p.ldhts + (pbase >> 5);
+            *(uint32_t *)dst = src[0];
+            if (t.row0 + 128 < t.end) *(uint32_t *)(dst + 4) = src[1];
         }
         return -1;
     }
@@ -671,7 +743,7 @@ struct WgradProblem {
         return p.bq + (int64_t)(t.n0 + r < p.Kout ? t.n0 + r : p.Kout - 1) * p.ldb;
     }
 
-    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
         if (t.slot >= 0) {  // one K slice: fp32 partial, laid out [sub-tile][thread]
             v4f *dst = (v4f *)p.ws + (int64_t)t.slot * (S::BM * S::BN / 4);
 #pragma unroll
@@ -850,14 +922,19 @@ extern "C" int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T,
                                 const int32_t *token_of, const uint8_t *wq, const uint8_t *ws, int64_t stride_we,
                                 int64_t ldw, int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
                                 uint8_t *hq, int64_t ldhq, uint8_t *hs, int64_t ldhs, void *pre, int64_t ldpre,
-                                int act_dtype, int64_t M, int64_t H, int64_t K, void *stream) {
+                                uint8_t *htq, int64_t ldhtq, uint8_t *hts, int64_t ldhts, int act_dtype, int64_t M,
+                                int64_t H, int64_t K, void *stream) {
     if (!sizes_ok(E, M, H, K) || H % MX_BLOCK || ldx < K || ldw < K || ldhq < H || ldhs < H / MX_BLOCK ||
-        (pre && ldpre < 2 * H) || !token_of)
+        (pre && ldpre < 2 * H) || (htq != nullptr) != (hts != nullptr))
         return MX_EINVAL;
+    const int64_t mpad = ((M + 127) / 128 + E) * 128;
+    if (htq && (ldhtq < mpad - 128 * E || ldhts < (mpad - 128 * E) / MX_BLOCK)) return MX_EINVAL;
     if (M == 0 || H == 0) return MX_OK;
     GroupedArgs a = base_args(xq, xs, ldx, ldxs, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
     a.hq = hq, a.ldhq = ldhq, a.hs = hs, a.ldhs = ldhs, a.pre = pre, a.ldpre = ldpre;
-    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 8) || ldpre % 4)))
+    a.htq = htq, a.ldhtq = ldhtq, a.hts = hts, a.ldhts = ldhts;
+    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 8) || ldpre % 4)) ||
+        (htq && (!aligned(htq, 16) || ldhtq % 16 || !aligned(hts, 4) || ldhts % 4)))
         return MX_EUNSUPPORTED;
     return launch_grouped_dt<MODE_GEMM1>(act_dtype, a, (hipStream_t)stream);
 }

@@ -67,6 +67,40 @@ def swiglu_bwd_mx_dual(dh: torch.Tensor, gu: torch.Tensor):
     return q, s, qt, st
 
 
+_WHOLE_RANGE: dict = {}
+
+
+def _whole_range(device, rows: int) -> torch.Tensor:
+    """``[0, rows]`` as the offset table of a single "expert" that owns every row (cached: built once)."""
+    key = (device, rows)
+    if key not in _WHOLE_RANGE:
+        _WHOLE_RANGE[key] = torch.tensor([0, rows], dtype=torch.int32, device=device)
+    return _WHOLE_RANGE[key]
+
+
+def fused_swiglu_projection(xq, xs, wq, ws, out_dtype):
+    """``gu = x . w_in^T`` with SwiGLU and both casts of ``h`` in the GEMM's epilogue.
+
+    Returns ``gu (M, 2H)`` in ``out_dtype`` (the rounded accumulators, saved for the backward),
+    ``h`` quantized along H ``(hq, hs)`` and along the tokens ``(htq, hts)``.  ``h`` is computed
+    from the rounded ``gu``, exactly as :func:`swiglu_mx_dual` does on the stored tensor.
+    Needs ``M % 128 == 0`` (token-axis tiles) and a 128-multiple contraction.
+    """
+    from kohakuwullm_amd.kernels.mxfp8.moe import launch_gemm1
+
+    m, k = xq.shape
+    hidden = wq.shape[0] // 2
+    dev = xq.device
+    gu = torch.empty(m, 2 * hidden, device=dev, dtype=out_dtype)
+    hq = torch.empty(m, hidden, device=dev, dtype=_FP8)
+    hs = torch.empty(m, hidden // BLOCK_SCALE, device=dev, dtype=torch.uint8)
+    htq = torch.empty(hidden, m, device=dev, dtype=_FP8)
+    hts = torch.empty(hidden, m // BLOCK_SCALE, device=dev, dtype=torch.uint8)
+    launch_gemm1(xq, xs, None, wq.unsqueeze(0), ws.unsqueeze(0), hq, hs, gu, _whole_range(dev, m), hidden, k, out_dtype,
+                 htq, hts)
+    return gu, hq, hs, htq, hts
+
+
 class _MXFP8SwiGLUMLP(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w_in, w_out, in_f, in_d, out_f, out_d):
@@ -76,6 +110,9 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         if x2d.stride(-1) != 1:
             x2d = x2d.contiguous()
         xq, xs, xtq, xts = quantize_mx_dual(x2d)
+        # GEMM, then one bandwidth-bound pass for SwiGLU and both casts: measured faster at the
+        # benchmark shape (220 + 89 us) than the same work in the GEMM's epilogue
+        # (fused_swiglu_projection: 329 us), whose vector ALU work cannot overlap the MFMAs.
         gu = mxfp8_matmul_pq(xq, xs, *in_f, compute)
         hq, hs, htq, hts = swiglu_mx_dual(gu)
         y = mxfp8_matmul_pq(hq, hs, *out_f, compute)

@@ -19,6 +19,7 @@ from kohakuwullm_amd import _lib
 from kohakuwullm_amd.kernels.mxfp8.grouped import (
     grouped_mxfp8_gemm,
     grouped_mxfp8_wgrad,
+    padded_rows,
     quantize_mx_cols_grouped,
 )
 from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE, quantize_mx, quantize_mx_cols
@@ -74,13 +75,20 @@ def _w_args(wq, ws):
     return (wq.data_ptr(), ws.data_ptr(), wq.stride(0), wq.stride(1), ws.stride(0), ws.stride(1))
 
 
-def launch_gemm1(xq, xs, token_of, wq, ws, hq, hs, pre, offsets, hidden, dim, act_dtype) -> None:
-    m = token_of.numel()
+def launch_gemm1(xq, xs, token_of, wq, ws, hq, hs, pre, offsets, hidden, dim, act_dtype, htq=None, hts=None) -> None:
+    """GEMM1 with its epilogue; ``token_of=None`` reads row m of ``xq`` for sorted row m.
+
+    ``htq``/``hts`` ``(H, Mpad)``/``(H, Mpad//32)``, when given, receive ``h`` quantized along the tokens.
+    """
+    m = hq.shape[0]
     _lib.invoke(
         "mx_experts_gemm1", 2.0 * m * 2 * hidden * dim, xq,
-        xq.data_ptr(), xs.data_ptr(), xq.shape[0], xq.stride(0), xs.stride(0), token_of.data_ptr(), *_w_args(wq, ws),
+        xq.data_ptr(), xs.data_ptr(), xq.shape[0], xq.stride(0), xs.stride(0),
+        0 if token_of is None else token_of.data_ptr(), *_w_args(wq, ws),
         offsets.data_ptr(), wq.shape[0], hq.data_ptr(), hq.stride(0), hs.data_ptr(), hs.stride(0),
         0 if pre is None else pre.data_ptr(), 0 if pre is None else pre.stride(0),
+        0 if htq is None else htq.data_ptr(), 0 if htq is None else htq.stride(0),
+        0 if hts is None else hts.data_ptr(), 0 if hts is None else hts.stride(0),
         _lib.MX_DTYPE[act_dtype], m, hidden, dim,
     )
 
@@ -156,19 +164,25 @@ class _MXFP8Experts(torch.autograd.Function):
         hq = torch.empty(m, hidden, device=x.device, dtype=_FP8)
         hs = torch.empty(m, hidden // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
         pre = torch.empty(m, 2 * hidden, device=x.device, dtype=x.dtype) if needs_grad else None
-        launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hidden, dim, x.dtype)
+        htq = hts = None
+        if ctx.needs_input_grad[2]:
+            # h along the tokens, for dW_out: written by GEMM1's epilogue instead of a pass over `pre`
+            mpad = padded_rows(m, packed.in_fwd[0].shape[0])
+            htq = torch.empty(hidden, mpad, device=x.device, dtype=_FP8)
+            hts = torch.empty(hidden, mpad // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+        launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hidden, dim, x.dtype, htq, hts)
         # pairs per token when `order` is the pair index token * top_k + slot; 0 = unknown layout
         top_k = gate.numel() // rows if rows and gate.numel() % rows == 0 else 0
         out = _routed_product(hq, hs, *packed.out_fwd, token_of, order, gate, offsets, rows, top_k, x.dtype)
         if needs_grad:
-            ctx.save_for_backward(x, hq, hs, pre, gate, token_of, order, offsets)
+            ctx.save_for_backward(x, hq, hs, pre, gate, token_of, order, offsets, htq, hts)
             ctx.packed = packed
             ctx.shapes = (hidden, dim, m, rows, top_k)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        x, hq, hs, pre, gate, token_of, order, offsets = ctx.saved_tensors
+        x, hq, hs, pre, gate, token_of, order, offsets, htq, hts = ctx.saved_tensors
         packed = ctx.packed
         hidden, dim, m, rows, top_k = ctx.shapes
         dev = dout.device
@@ -186,7 +200,6 @@ class _MXFP8Experts(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             # dW_out[e] = (gate-scaled dout rows of e).T @ h rows of e; h is rebuilt from `pre`
             dtq, dts = quantize_mx_cols_grouped(dout, offsets, m, index=token_of, row_scale=gate, scale_index=order)
-            htq, hts = quantize_mx_cols_grouped(pre, offsets, m, swiglu=True)
             dw_out = grouped_mxfp8_wgrad(dtq, dts, htq, hts, offsets, m, dout.dtype)
         if ctx.needs_input_grad[1]:
             # dW_in[e] = dpre rows of e .T @ x rows of e

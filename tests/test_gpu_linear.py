@@ -196,6 +196,22 @@ def test_fused_swiglu_mlp(oracle, tokens, dim, hidden):
     assert ora.rel_error(wo.grad.cpu(), wof.grad) < 0.12
 
 
+@pytest.mark.parametrize("tokens,dim,hidden", [(384, 256, 160), (128, 128, 32), (512, 384, 256)])
+def test_fused_swiglu_projection_equals_gemm_then_quantizer(tokens, dim, hidden):
+    """The first projection with SwiGLU and both casts in its epilogue == GEMM, then the fused quantizer."""
+    from kohakuwullm_amd.kernels.mxfp8.mlp import fused_swiglu_projection, swiglu_mx_dual
+    from kohakuwullm_amd.kernels.mxfp8.quantize import mxfp8_matmul_pq, quantize_mx
+
+    x, w_in = _draw(((tokens, dim), 1.0), ((2 * hidden, dim), 0.05))
+    xq, xs = quantize_mx(x.to(DEV))
+    wq, ws = quantize_mx(w_in.to(DEV))
+    gu, hq, hs, htq, hts = fused_swiglu_projection(xq, xs, wq, ws, torch.bfloat16)
+    gu_ref = mxfp8_matmul_pq(xq, xs, wq, ws)
+    assert torch.equal(gu, gu_ref)
+    for got, ref in zip((hq, hs, htq, hts), swiglu_mx_dual(gu_ref)):
+        assert got.shape == ref.shape and torch.equal(got.view(torch.uint8), ref.view(torch.uint8))
+
+
 def test_swiglu_dual_kernels_bitwise_vs_composition(oracle):
     """The fused SwiGLU quantizers equal quantizing the separately computed activation."""
     from kohakuwullm_amd.kernels.mxfp8.mlp import swiglu_bwd_mx_dual, swiglu_mx_dual

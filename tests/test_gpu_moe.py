@@ -314,7 +314,23 @@ def test_gemm1_intermediates(oracle):
     hq = torch.zeros(m, hid, device=DEV, dtype=F8)
     hs = torch.zeros(m, hid // 32, device=DEV, dtype=torch.uint8)
     pre = torch.zeros(m, 2 * hid, device=DEV, dtype=torch.bfloat16)
-    launch_gemm1(xq, xs, token_of.to(DEV), *packed.in_fwd, hq, hs, pre, offsets.to(DEV), hid, dim, torch.bfloat16)
+    from kohakuwullm_amd.kernels.mxfp8.grouped import padded_rows, quantize_mx_cols_grouped
+
+    mpad = padded_rows(m, e)
+    htq = torch.zeros(hid, mpad, device=DEV, dtype=F8)
+    hts = torch.zeros(hid, mpad // 32, device=DEV, dtype=torch.uint8)
+    launch_gemm1(xq, xs, token_of.to(DEV), *packed.in_fwd, hq, hs, pre, offsets.to(DEV), hid, dim, torch.bfloat16, htq, hts)
+    # the token-axis copy written by the epilogue is the grouped quantizer's result on the stored pre, bit for bit
+    rq, rs = quantize_mx_cols_grouped(pre, offsets.to(DEV), m, swiglu=True)
+    valid = torch.zeros(mpad, dtype=torch.bool)
+    pos = 0
+    for c in counts:
+        tiles = -(-c // 128)
+        valid[pos : pos + tiles * 128] = True
+        pos += tiles * 128
+    assert torch.equal(htq.view(torch.uint8).cpu()[:, valid], rq.view(torch.uint8).cpu()[:, valid])
+    assert torch.equal(hts.cpu()[:, valid.view(-1, 32)[:, 0]], rs.cpu()[:, valid.view(-1, 32)[:, 0]])
+    assert not htq.view(torch.uint8).cpu()[:, ~valid].any()  # nothing is written past the experts' tiles
     assert oracle.rel_error(pre.cpu(), ref["pre"].double()) < 2e-3  # same bf16 values up to accumulation-order ulps
     hd = oracle.dequant(hq.view(torch.uint8).cpu(), hs.cpu())
     assert oracle.rel_error(hd, oracle.dequant(ref["hq"], ref["hs"])) < 2e-2
