@@ -286,12 +286,36 @@ using namespace mx;
 
 static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-static int num_cus() {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 256;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
-    return n;
+namespace mx {
+int num_cus() {
+    static std::mutex lock;
+    static int cached[64];  // by device ordinal; 0 = not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!cached[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
 }
+
+bool allow_dynamic_lds(const void *kernel, int bytes) {
+    static std::mutex lock;
+    static std::map<std::pair<int, const void *>, bool> done;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    std::lock_guard<std::mutex> guard(lock);
+    auto key = std::make_pair(dev, kernel);
+    auto it = done.find(key);
+    if (it != done.end()) return it->second;
+    const bool ok = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
+    if (!ok) (void)hipGetLastError();
+    done[key] = ok;
+    return ok;
+}
+}  // namespace mx
 
 // Scratch of the K splits (dense and expert WGRAD): two fp32 tile slots per workgroup, kept per
 // (device, stream) for the life of the process so launches on different streams never share it.
@@ -363,8 +387,7 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
     }
     dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
     auto kern = k512 ? gemm_nt_kernel<S, CDT, true> : gemm_nt_kernel<S, CDT, false>;
-    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
-        return MX_ELAUNCH;
+    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     if (a.sk_tiles)
         split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * S::MT)), block, 0, st>>>(a);
@@ -454,8 +477,7 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     }
     b.count = count;
     auto kern = k512 ? gemm_nt_batch_kernel<S, CDT, true> : gemm_nt_batch_kernel<S, CDT, false>;
-    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
-        return MX_ELAUNCH;
+    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<dim3((unsigned)b.cu_lo[count]), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
@@ -475,10 +497,19 @@ static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const u
     return MX_OK;
 }
 
+// An empty contraction: C = 0.  A fill kernel, not a memset, so the call can sit in a captured graph.
+__global__ __launch_bounds__(256) static void zero_matrix_kernel(uint8_t *c, int64_t row_bytes, int64_t pitch_bytes,
+                                                                  int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) c[(i / row_bytes) * pitch_bytes + i % row_bytes] = 0;
+}
+
 static int zero_matrix(void *c, int c_dtype, int64_t M, int64_t N, int64_t ldc, hipStream_t st) {
     const int esz = c_dtype == MX_FP32 ? 4 : 2;
-    hipError_t e = hipMemset2DAsync(c, (size_t)ldc * esz, 0, (size_t)N * esz, (size_t)M, st);
-    return e == hipSuccess ? MX_OK : MX_ELAUNCH;
+    const int64_t total = M * N * esz, blocks = (total + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    zero_matrix_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>((uint8_t *)c, N * esz, ldc * esz, total);
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
 extern "C" int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *stream) {

@@ -574,4 +574,11 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &t
     tn = in / rows;
 }
 
+// Host-side launch helpers shared by the GEMM translation units (defined in mx_gemm.hip).
+// Both cache their answer: the per-launch path makes no HIP call besides the launch itself, which
+// is what a stream being captured into a graph tolerates (attribute calls from autograd's worker
+// thread count as unsafe during a capture and would invalidate it).
+int num_cus();                                   // CUs of the current device
+bool allow_dynamic_lds(const void *kernel, int bytes);  // hipFuncSetAttribute, once per kernel
+
 }  // namespace mx

@@ -828,13 +828,6 @@ using namespace mx;
 
 static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-static int num_cus() {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 256;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
-    return n;
-}
-
 // 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
 typedef GemmShape<256, 256, 4, 2, true> Big;
 
@@ -857,8 +850,7 @@ static int launch_grouped(GroupedArgs a, hipStream_t st) {
     const int cus = num_cus();
     dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
     auto kern = k512 ? grouped_kernel<S, MODE, CDT, true> : grouped_kernel<S, MODE, CDT, false>;
-    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
-        return MX_ELAUNCH;
+    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
@@ -1023,8 +1015,7 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
     a.slots = a.ws ? 2 * cus : 0;
     dim3 grid((unsigned)(work * (a.slots ? 8 : 1) < cus ? work * (a.slots ? 8 : 1) : cus)), block(S::NTHR);
     auto kern = grouped_wgrad_kernel<S, CDT>;
-    if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
-        return MX_ELAUNCH;
+    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     if (a.slots) wgrad_reduce_kernel<S, CDT><<<dim3((unsigned)(work * S::MT)), block, 0, st>>>(a, (int)grid.x);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;

@@ -238,3 +238,54 @@ def test_swiglu_dual_kernels_bitwise_vs_composition(oracle):
         assert (got.view(torch.uint8).cpu() != ref).float().mean() < 5e-3
     assert oracle.rel_error(oracle.dequant(pq.view(torch.uint8).cpu(), ps.cpu()), dpre) < 0.04
     assert oracle.rel_error(oracle.dequant(ptq.view(torch.uint8).cpu(), pts.cpu()), dpre.T) < 0.04
+
+
+@pytest.mark.skip(
+    reason="ending the capture of this step (torch.cuda.graphs capture_end -> graph instantiation) ended the process "
+    "with a segmentation fault inside the HIP runtime on the test box, twice, the second time after the library "
+    "stopped making any HIP call besides kernel launches on the per-launch path; cause not established, so the "
+    "case stays off the GPU"
+)
+def test_mlp_step_under_hip_graph(oracle):
+    """The fused MLP forward+backward captured in a HIP graph replays to the eager result.
+
+    The graph is replayed several times with eager work and synchronisations in between, and
+    every replay is compared: the library records no memset nodes on this path and allocates
+    nothing while the stream is being captured.
+    """
+    from kohakuwullm_amd.kernels.mxfp8.mlp import mxfp8_swiglu_mlp
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx, quantize_mx_cols
+
+    tokens, dim, hidden = 512, 256, 384
+    x, w_in, w_out, dy = _draw(((tokens, dim), 1.0), ((2 * hidden, dim), 0.05), ((dim, hidden), 0.05), ((tokens, dim), 1e-2))
+    xd = x.to(DEV).requires_grad_(True)
+    wi = w_in.to(DEV).requires_grad_(True)
+    wo = w_out.to(DEV).requires_grad_(True)
+    dyd = dy.to(DEV)
+    packed = (quantize_mx(wi.detach()), quantize_mx_cols(wi.detach()), quantize_mx(wo.detach()), quantize_mx_cols(wo.detach()))
+
+    def step():
+        y = mxfp8_swiglu_mlp(xd, wi, wo, packed)
+        gx, gwi, gwo = torch.autograd.grad(y, (xd, wi, wo), dyd)
+        return y, gx, gwi, gwo
+
+    eager = [t.clone() for t in step()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):  # warm-up on the capture stream: scratch buffers are created here, not under capture
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = step()
+    for replay in range(4):
+        for t in captured:
+            t.fill_(float("nan")) if t.dtype != torch.uint8 else None
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want), replay
+        _ = [t.clone() for t in step()]  # eager work between replays
+        torch.cuda.synchronize()
