@@ -118,17 +118,6 @@ struct DenseProblem {
         c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
     }
 
-    // Address of K byte 0 of row r of the tile's [A rows; B rows] list.
-    __device__ __forceinline__ const uint8_t *line(const Tile &t, int r) const {
-        if (r < S::BM) {
-            const int mrem = p.M - t.m0;
-            return p.aq + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.lda;
-        }
-        r = b_row_of_lds<S>(r - S::BM);
-        const int nrem = p.N - t.n0;
-        return p.bq + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldb;
-    }
-
     static_assert(S::LANES_N, "the dense kernels use the layout that puts neighbouring lanes on neighbouring N");
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 

@@ -32,10 +32,6 @@
 
 #include "mx_common.h"
 
-#ifndef MX_L2_AHEAD
-#define MX_L2_AHEAD 0
-#endif
-
 namespace mx {
 
 typedef __attribute__((address_space(1))) const void gptr_t;
@@ -45,20 +41,14 @@ typedef __attribute__((address_space(3))) void lptr_t;
 // plus the lane's 32-bit byte offset is the global address; the wave's 64 x 16 bytes land
 // contiguously in LDS at byte address `lds` (wave-uniform, goes through M0).
 // Written as inline asm on purpose: the kernel orders these copies against LDS reads itself,
-// with explicit vmcnt waits and workgroup barriers, and lets chosen younger operations (L2
-// touches, epilogue stores) stay in flight across a barrier; the compiler's own accounting
-// would insert a full vmcnt(0) before every LDS read that follows a copy it can see.
+// with explicit vmcnt waits and workgroup barriers, and lets chosen younger operations (the
+// epilogue's stores) stay in flight across a barrier; the compiler's own accounting would
+// insert a full vmcnt(0) before every LDS read that follows a copy it can see.
 __device__ __forceinline__ void dma16(const uint8_t *base, uint32_t voff, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(base), "s"(lds)
                  : "memory");
-}
-
-// One 4-byte direct-to-LDS load per lane whose only purpose is to pull the 128-byte line at
-// `g` into L2 ahead of the stage that needs it; the 256 bytes it deposits in LDS are junk.
-__device__ __forceinline__ void l2_touch(const uint8_t *g, uint32_t lds_junk) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(lds_junk) : "memory");
 }
 
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
@@ -98,7 +88,7 @@ struct GemmShape {
     // a wave (16 rows x 4 planes) read 64 different banks.
     static constexpr int PA = BM + 16, PB = LANES_N ? BN + 16 : BN + 32;
     static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
-    static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B) + NW * 256;
+    static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B);
     static constexpr bool TWO_ROWS = BM + BN > NTHR;
     static_assert(LANES_N || WTN % 64 == 0, "a wave's N extent must be a multiple of 64");
     static_assert(!LANES_N || NT == 8, "8 sub-tiles along N give a lane 8 consecutive N: one 16-byte store");
@@ -371,8 +361,6 @@ struct LdsScratch {
 //   bool P::next(Tile &t)                   advance to this workgroup's next tile (false = done);
 //                                           tiles with an empty K range are finished inside next()
 //   void P::context(const Tile &, const Lane &, IssueCtx<S> &)
-//   const uint8_t *P::line(const Tile &, int operand_row)   address of K byte 0 of row
-//                                           operand_row of the [A rows; B rows] list (for L2 touches)
 //   int  P::epilogue(const Tile &, const Lane &, v4f (&acc)[MT][NT], const LdsScratch &)   returns how many stores each
 //                                           lane issued if that number is the same compile-time
 //                                           constant P::NST for the whole wave, else -1
@@ -383,12 +371,10 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     uint8_t *const ldsB = smem + 2 * S::DATA_A;                                  // [2][BN*128]
     uint32_t *const ldsSA = (uint32_t *)(smem + 2 * (S::DATA_A + S::DATA_B));    // [2][4][PA]
     uint32_t *const ldsSB = ldsSA + 2 * 4 * S::PA;                               // [2][4][PB]
-    uint8_t *const ldsJunk = (uint8_t *)(ldsSB + 2 * 4 * S::PB);                 // [NW][256]
 
     const Lane L = lane_of<S>();
     const bool has_row0 = L.tid < S::BM + S::BN;
     const int kb_end = prob.kb_end;
-    constexpr int AHEAD = MX_L2_AHEAD;  // L2 touches run this many stages ahead of the copy engine (0 = off)
 
     // per-lane LDS read offsets: low half = 16-byte chunk g, high half = chunk g + 4 (= offset ^ 64)
     const int a_row = L.wm * S::WTM + L.r16;
@@ -402,20 +388,6 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     IssueCtx<S> ctx;
     prob.context(cur, L, ctx);
 
-    // Lines of stage `k` (relative to the current tile's first stage) that this wave touches:
-    // row tid of the [A rows; B rows] list.  Stages past the tile's end belong to the next tile.
-    auto touch = [&](int k, int KT) -> bool {
-        // every wave issues it (threads past the row list repeat the last row): the stage-end
-        // wait counts on exactly one operation younger than the stage's copies
-        const int r = L.tid < S::BM + S::BN ? L.tid : S::BM + S::BN - 1;
-        const uint8_t *g;
-        if (k < KT) g = prob.line(cur, r) + (int64_t)(cur.kt0 + k) * 128;
-        else if (has_next && k - KT < nxt.kt1 - nxt.kt0) g = prob.line(nxt, r) + (int64_t)(nxt.kt0 + k - KT) * 128;
-        else return false;
-        l2_touch(g, __builtin_amdgcn_readfirstlane(lds_addr(ldsJunk) + L.wave * 256));
-        return true;
-    };
-
     int gstage = 0;  // stages issued so far, over all tiles: LDS data buffer = gstage & 1
     int gsuper = 0;  // super-steps so far: LDS scale buffer = gsuper & 1
 
@@ -425,7 +397,6 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);
         if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);
         issue_stage<S>(ctx, L, ctx.kt0, ldsA, ldsB, 0);
-        for (int k = 1; k <= AHEAD; k++) touch(k, ctx.kt1 - ctx.kt0);
         if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
         if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
     }
@@ -452,8 +423,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
                 sb[j] = (int)ldsSB[(sbuf * 4 + L.g) * S::PB + b_row + (S::LANES_N ? 16 * j : b_sub_off(j))];
 
             // One K stage.  In every stage but the tile's last, the next stage's operands are
-            // put in flight first, then the L2 touch for the stage AHEAD beyond it, which is the
-            // only vector-memory operation allowed to stay in flight across the stage's end.
+            // put in flight during the stage and waited for at its end.
             // In the last stage nothing of this tile is left to fetch, so the copy context is
             // switched to the next tile and ITS first stage and scales go in flight; the wait
             // and barrier that publish them come after the epilogue.
@@ -463,7 +433,6 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         if (k < KT) {                                                                                         \
             const int buf = gstage & 1;                                                                       \
             const bool last = k + 1 == KT;                                                                    \
-            bool touched = false;                                                                             \
             int kt_issue = kt0 + k + 1;                                                                       \
             if (!last) {                                                                                      \
                 if (SIDX == 3) {                                                                              \
@@ -485,9 +454,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             compute_stage<S, SIDX>(ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64, b_rd,     \
                                    b_rd ^ 64, sa, sb, acc, ctx, L, kt_issue, ldsA, ldsB, buf ^ 1);            \
             if (!last) {                                                                                      \
-                touched = AHEAD && touch(k + 1 + AHEAD, KT);                                                  \
-                if (touched) wait_vm_allow(1);                                                                \
-                else wait_vm_allow(0);                                                                        \
+                wait_vm_allow(0);                                                                             \
                 __syncthreads();                                                                              \
             }                                                                                                 \
             gstage++;                                                                                         \
@@ -502,7 +469,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         }
         // The next tile's first stage and scales are already in flight: the epilogue's
         // conversions run under that latency, and when every lane issued the same known number
-        // of stores the wait lets exactly those (and the L2 touch before them) stay in flight,
+        // of stores the wait lets exactly those stay in flight,
         // so the stores drain under the next tile's first stage.
         const int lastbuf = (gstage - 1) & 1;
         const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B});
@@ -511,9 +478,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);
         }
         if (!has_next) break;
-        const bool touched = AHEAD && stores == P::NST && touch(KT + AHEAD, KT);
-        if (stores == P::NST && touched) wait_vm_allow_c<P::NST + 1>();
-        else if (stores == P::NST) wait_vm_allow_c<P::NST>();
+        if (stores == P::NST) wait_vm_allow_c<P::NST>();
         else wait_vm_allow(0);
         __syncthreads();
         cur = nxt;

@@ -242,11 +242,6 @@ struct GroupedProblem {
         c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
     }
 
-    __device__ __forceinline__ const uint8_t *line(const Tile &t, int r) const {
-        if (r < S::BM) return p.xq + (int64_t)a_src_row(t, r) * p.ldx;
-        return p.wq + (int64_t)t.expert * p.stride_we + (int64_t)b_src_row(t, r - S::BM) * p.ldw;
-    }
-
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT],
                                             const LdsScratch &lds) const {
         if constexpr (MODE == MODE_PLAIN) return epilogue_plain(t, L, acc);
@@ -735,12 +730,6 @@ struct WgradProblem {
         };
         c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
         c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
-    }
-
-    __device__ __forceinline__ const uint8_t *line(const Tile &t, int r) const {
-        if (r < S::BM) return p.aq + (int64_t)(t.m0 + r < p.N ? t.m0 + r : p.N - 1) * p.lda;
-        r = b_row_of_lds<S>(r - S::BM);
-        return p.bq + (int64_t)(t.n0 + r < p.Kout ? t.n0 + r : p.Kout - 1) * p.ldb;
     }
 
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
