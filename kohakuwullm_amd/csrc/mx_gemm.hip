@@ -21,6 +21,8 @@ struct DenseArgs {
     int c_vec;
     int accumulate;  // fp32 atomic add into C (split-K)
     int split_k;     // number of K slices; tile ids run over tiles_m * tiles_n * split_k
+    float *slice_ws;  // with split_k > 1 and no accumulate: slice s of tile i leaves its fp32 partial in slot
+                      // i * split_k + s of this buffer and slice_reduce_kernel adds the slices
     // Even K split of the last, partial round of tiles.  Tile ids [0, dp_tiles) are whole tiles
     // dealt round-robin; the K stages of the remaining sk_tiles tiles are laid end to end (each
     // tile padded to KT4 stages) and cut into gridDim.x equal ranges of sk_q stages, one per
@@ -36,7 +38,8 @@ template <typename S, int CDT>
 struct DenseProblem {
     struct Tile {
         int m0, n0, kt0, kt1;
-        int sk;  // index among the K-split tiles when this unit is one piece of several, else -1
+        int sk;    // index among the K-split tiles when this unit is one piece of several, else -1
+        int slot;  // slot of slice_ws this K slice is written to, else -1
     };
     const DenseArgs p;  // a copy: its fields live in scalar registers, never re-read through a pointer
     int next_id;
@@ -66,6 +69,7 @@ struct DenseProblem {
             t.kt0 = k0;
             t.kt1 = stop < KT ? stop : KT;
             t.sk = (k0 == 0 && stop >= KT) ? -1 : local;
+            t.slot = -1;
             sk_pos += (stop < KT4 ? stop : KT4) - k0;
             return true;
         }
@@ -73,8 +77,10 @@ struct DenseProblem {
         if (p.sk_tiles && next_id >= p.dp_tiles) return false;
         if (next_id >= per_slice * p.split_k) return false;
         const int slice = next_id / per_slice;
+        const int index = next_id - slice * per_slice;
         int tm, tn;
-        tile_of(next_id - slice * per_slice, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of(index, p.tiles_m, p.tiles_n, tm, tn);
+        t.slot = p.slice_ws ? index * p.split_k + slice : -1;
         t.m0 = tm * S::BM;
         t.n0 = tn * S::BN;
         const int KT = p.K >> 7;
@@ -143,6 +149,14 @@ struct DenseProblem {
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
         if (t.sk >= 0) {
             write_piece(t, L, acc);
+            return -1;
+        }
+        if (t.slot >= 0) {
+            v4f *dst = (v4f *)p.slice_ws + (int64_t)t.slot * (S::BM * S::BN / 4);
+#pragma unroll
+            for (int i = 0; i < S::MT; i++)
+#pragma unroll
+                for (int j = 0; j < S::NT; j++) dst[(i * S::NT + j) * S::NTHR + L.tid] = acc[i][j];
             return -1;
         }
         // Interior tiles of a vector-aligned C store unconditionally: every lane issues NST stores.
@@ -234,6 +248,35 @@ __global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
             const v4f lo = {sum[0][v], sum[1][v], sum[2][v], sum[3][v]};
             const v4f hi = {sum[4][v], sum[5][v], sum[6][v], sum[7][v]};
             store8<CDT>(p.c, (int64_t)m * p.ldc + n, lo, hi, nvalid, p.c_vec != 0);
+        }
+    }
+}
+
+// Adds the split_k fp32 slices of every tile, in slice order, and stores C.  One block per (tile, i).
+template <typename S, int CDT>
+__global__ __launch_bounds__(S::NTHR) void slice_reduce_kernel(DenseArgs p) {
+    const int index = blockIdx.x / S::MT, i = blockIdx.x % S::MT;
+    const int tid = threadIdx.x;
+    v4f sum[S::NT];
+#pragma unroll
+    for (int j = 0; j < S::NT; j++) sum[j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int sl = 0; sl < p.split_k; sl++) {
+        const v4f *src = (const v4f *)p.slice_ws + (int64_t)(index * p.split_k + sl) * (S::BM * S::BN / 4);
+#pragma unroll
+        for (int j = 0; j < S::NT; j++) sum[j] += src[(i * S::NT + j) * S::NTHR + tid];
+    }
+    int tm, tn;
+    tile_of(index, p.tiles_m, p.tiles_n, tm, tn);
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave / S::WGN, wn = wave % S::WGN;
+    const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int m = tm * S::BM + wm * S::WTM + 16 * i + 4 * (lane >> 4) + v;
+        if (m < p.M && n < p.N) {
+            const v4f lo = {sum[0][v], sum[1][v], sum[2][v], sum[3][v]};
+            const v4f hi = {sum[4][v], sum[5][v], sum[6][v], sum[7][v]};
+            store8<CDT>(p.c, (int64_t)m * p.ldc + n, lo, hi, p.N - n < 8 ? p.N - n : 8, p.c_vec != 0);
         }
     }
 }
@@ -411,7 +454,11 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
 // Several products behind one launch, the workgroups shared out among them in groups of 8 (one
 // per XCD, so each problem's tile order keeps its XCD locality).  A group goes, one at a time,
 // to the problem that would otherwise finish last; cost of a problem on n workgroups =
-// rounds of tiles x (K stages + 4 for the tile's prologue and epilogue).
+// rounds of tiles x (K stages + 4 for the tile's prologue and epilogue).  A problem with few,
+// long tiles (a weight gradient) may in addition be cut into 2 or 4 K slices that run as
+// independent tiles and leave fp32 partial sums for slice_reduce_kernel; every combination of
+// slice counts is priced (a partial tile costs about 0.1 stage of everyone's time) and the
+// cheapest plan wins, against running the products one after the other as well.
 template <int CDT>
 static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     typedef DenseShape S;
@@ -419,8 +466,8 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     const int groups = cus / 8;
     bool fuse = count > 1 && count <= MX_BATCH_MAX && groups >= count && split_mode();
     DenseBatchArgs b;
-    int64_t tiles[MX_BATCH_MAX], cost[MX_BATCH_MAX], alone = 0;
-    int share[MX_BATCH_MAX];
+    int64_t tiles[MX_BATCH_MAX], alone = 0;
+    int KT[MX_BATCH_MAX];
     bool k512 = true;
     for (int j = 0; j < count && fuse; j++) {
         DenseArgs &a = probs[j];
@@ -434,28 +481,55 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         a.dp_tiles = a.tiles_m * a.tiles_n, a.sk_tiles = 0, a.sk_q = 0, a.sk_ws = nullptr;
         k512 = k512 && a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0;
         tiles[j] = a.dp_tiles;
-        cost[j] = (a.K >> 7) + 4;
-        share[j] = 1;
-        alone += (tiles[j] + cus - 1) / cus * cost[j];
-        b.prob[j] = a;
+        KT[j] = a.K >> 7;
+        alone += (tiles[j] + cus - 1) / cus * (KT[j] + 4);
     }
+    int share[MX_BATCH_MAX], slices[MX_BATCH_MAX], best_share[MX_BATCH_MAX], best_slices[MX_BATCH_MAX];
+    int64_t best = -1;
     if (fuse) {
-        auto finish = [&](int j) { return (tiles[j] + 8 * share[j] - 1) / (8 * share[j]) * cost[j]; };
-        for (int left = groups - count; left > 0; left--) {
-            int worst = -1;
-            for (int j = 0; j < count; j++)
-                if (8 * share[j] < tiles[j] && (worst < 0 || finish(j) > finish(worst))) worst = j;
-            if (worst < 0) break;
-            share[worst]++;
+        const int slots = 2 * cus;  // fp32 tile slots of the scratch
+        auto per_slice = [&](int j) { return (((KT[j] + slices[j] - 1) / slices[j]) + 3) & ~3; };
+        auto units = [&](int j) { return tiles[j] * slices[j]; };
+        auto finish = [&](int j) { return (units(j) + 8 * share[j] - 1) / (8 * share[j]) * (per_slice(j) + 4); };
+        int combos = 1;
+        for (int j = 0; j < count; j++) combos *= 3;
+        for (int code = 0; code < combos; code++) {
+            int64_t partial = 0;
+            bool ok = true;
+            for (int j = 0, c = code; j < count; j++, c /= 3) {
+                slices[j] = 1 << (c % 3);
+                // every slice must own K stages, and at least 16 of them to be worth a partial tile
+                if (slices[j] > 1 && (KT[j] < 16 * slices[j] || (slices[j] - 1) * per_slice(j) >= KT[j])) ok = false;
+                if (slices[j] > 1) partial += units(j);
+                share[j] = 1;
+            }
+            if (!ok || partial > slots) continue;
+            for (int left = groups - count; left > 0; left--) {
+                int worst = -1;
+                for (int j = 0; j < count; j++)
+                    if (8 * share[j] < units(j) && (worst < 0 || finish(j) > finish(worst))) worst = j;
+                if (worst < 0) break;
+                share[worst]++;
+            }
+            int64_t together = partial ? 4 + partial / 10 : 0;
+            int64_t longest = 0;
+            for (int j = 0; j < count; j++) longest = finish(j) > longest ? finish(j) : longest;
+            together += longest;
+            if (best < 0 || together < best) {
+                best = together;
+                for (int j = 0; j < count; j++) best_share[j] = share[j], best_slices[j] = slices[j];
+            }
         }
-        int64_t together = 0;
-        b.cu_lo[0] = 0;
-        for (int j = 0; j < count; j++) {
-            together = finish(j) > together ? finish(j) : together;
-            const int64_t wgs = 8 * share[j] < tiles[j] ? 8 * share[j] : tiles[j];
-            b.cu_lo[j + 1] = b.cu_lo[j] + (int)wgs;
+        fuse = best >= 0 && best < alone;
+    }
+    float *scratch = nullptr;
+    if (fuse) {
+        bool any = false;
+        for (int j = 0; j < count; j++) any = any || best_slices[j] > 1;
+        if (any) {
+            scratch = split_scratch(st, cus, (size_t)S::BM * S::BN);
+            if (!scratch) fuse = false;  // no scratch (allocation failed or the stream is being captured)
         }
-        fuse = together < alone;
     }
     if (!fuse) {
         for (int j = 0; j < count; j++) {
@@ -464,10 +538,27 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         }
         return MX_OK;
     }
+    b.cu_lo[0] = 0;
+    int64_t slot_base = 0;
+    for (int j = 0; j < count; j++) {
+        DenseArgs &a = probs[j];
+        a.split_k = best_slices[j];
+        if (a.split_k > 1) {
+            a.slice_ws = scratch + slot_base * (S::BM * S::BN);
+            slot_base += tiles[j] * a.split_k;
+        }
+        const int64_t u = tiles[j] * a.split_k;
+        const int64_t wgs = 8 * best_share[j] < u ? 8 * best_share[j] : u;
+        b.cu_lo[j + 1] = b.cu_lo[j] + (int)wgs;
+        b.prob[j] = a;
+    }
     b.count = count;
     auto kern = k512 ? gemm_nt_batch_kernel<S, CDT, true> : gemm_nt_batch_kernel<S, CDT, false>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<dim3((unsigned)b.cu_lo[count]), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
+    for (int j = 0; j < count; j++)
+        if (probs[j].split_k > 1)
+            slice_reduce_kernel<S, CDT><<<dim3((unsigned)(tiles[j] * S::MT)), dim3(S::NTHR), 0, st>>>(probs[j]);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
@@ -480,6 +571,7 @@ static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const u
     a.M = (int)M, a.N = (int)N, a.K = (int)K;
     a.lda = lda, a.ldas = ldas, a.ldb = ldb, a.ldbs = ldbs, a.ldc = ldc;
     a.accumulate = 0, a.split_k = 1;
+    a.slice_ws = nullptr;
     a.tiles_m = a.tiles_n = a.c_vec = 0;
     a.dp_tiles = a.sk_tiles = a.sk_q = 0;
     a.sk_ws = nullptr;

@@ -63,7 +63,9 @@ def test_attention_fused_qkv_equals_slices(oracle, attn):
         # every output element contracts the same K sequence in the same order: identical bits
         assert torch.equal(yp, y[:, lo:hi])
         yp.backward(d_qkv[:, lo:hi].to(DEV))
-        assert torch.equal(part.weight.grad, fused.weight.grad[lo:hi])
+        # dW may be cut into a different number of K slices per launch plan: the same fp32 sum up to
+        # its order, then one bf16 rounding
+        assert oracle.rel_error(part.weight.grad.cpu(), fused.weight.grad[lo:hi].double().cpu()) < 2e-3
         dx_sum += xp.grad.float()
     # dX of the fused product contracts all 3072 output features at once; the three partial
     # dgrads are rounded to bf16 separately, so this one is a norm comparison
