@@ -49,7 +49,7 @@ struct DenseProblem {
 
     __device__ DenseProblem(const DenseArgs &args, int first_, int stride_)
         : p(args), next_id(first_), kb_end(args.K >> 5), first(first_), stride(stride_) {
-        const int KT4 = ((p.K >> 7) + 3) & ~3;
+        const int KT4 = ((((p.K + 127) >> 7)) + 3) & ~3;
         const int total = p.sk_tiles * KT4;
         sk_pos = first * p.sk_q;
         sk_end = sk_pos + p.sk_q < total ? sk_pos + p.sk_q : total;
@@ -58,7 +58,7 @@ struct DenseProblem {
     __device__ __forceinline__ bool next(Tile &t) {
         const int per_slice = p.tiles_m * p.tiles_n;
         if (sk_pos < sk_end) {
-            const int KT = p.K >> 7, KT4 = (KT + 3) & ~3;
+            const int KT = ((p.K + 127) >> 7), KT4 = (KT + 3) & ~3;
             const int local = sk_pos / KT4;
             const int k0 = sk_pos - local * KT4;
             const int stop = k0 + (sk_end - sk_pos);
@@ -83,7 +83,7 @@ struct DenseProblem {
         t.slot = p.slice_ws ? index * p.split_k + slice : -1;
         t.m0 = tm * S::BM;
         t.n0 = tn * S::BN;
-        const int KT = p.K >> 7;
+        const int KT = ((p.K + 127) >> 7);
         // K slices are multiples of 4 stages so every slice starts on a 16-byte scale boundary
         const int per = (((KT + p.split_k - 1) / p.split_k) + 3) & ~3;
         t.kt0 = slice * per < KT ? slice * per : KT;
@@ -99,6 +99,8 @@ struct DenseProblem {
         c.b_base = p.bq + (int64_t)t.n0 * p.ldb;
         c.kt0 = t.kt0;
         c.kt1 = t.kt1;
+        c.tail_bytes = p.K & 127;
+        c.tail_kt = c.tail_bytes ? p.K >> 7 : -1;
         const int mrem = p.M - t.m0, nrem = p.N - t.n0;
 #pragma unroll
         for (int q = 0; q < S::QA; q++) {
@@ -124,7 +126,6 @@ struct DenseProblem {
         c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
     }
 
-    static_assert(S::LANES_N, "the dense kernels use the layout that puts neighbouring lanes on neighbouring N");
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
     // Slot of workgroup `wg`'s piece of the split tile whose stages start at `begin` in the
@@ -138,7 +139,7 @@ struct DenseProblem {
     // One piece of a K-split tile: the fp32 accumulators go to the workgroup's slot, laid out
     // [sub-tile][thread] so the stores and the reduction kernel's loads are contiguous.
     __device__ __forceinline__ void write_piece(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
-        const int KT4 = ((p.K >> 7) + 3) & ~3;
+        const int KT4 = ((((p.K + 127) >> 7)) + 3) & ~3;
         v4f *mine = piece_slot(p, first, t.sk * KT4);
 #pragma unroll
         for (int i = 0; i < S::MT; i++)
@@ -188,7 +189,7 @@ struct DenseProblem {
     }
 };
 
-template <typename S, int CDT, bool K512>
+template <typename S, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
@@ -205,7 +206,7 @@ struct DenseBatchArgs {
     int count;
 };
 
-template <typename S, int CDT, bool K512>
+template <typename S, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     int j = 0;
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b
 // covered whole were stored by the GEMM itself.
 template <typename S, int CDT>
 __global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
-    const int KT = p.K >> 7, KT4 = (KT + 3) & ~3;
+    const int KT = ((p.K + 127) >> 7), KT4 = (KT + 3) & ~3;
     const int local = blockIdx.x / S::MT;
     const int i = blockIdx.x % S::MT;
     const int begin = local * KT4;
@@ -376,6 +377,13 @@ float *split_scratch(hipStream_t st, int cus, size_t tile_floats) {
 }
 }  // namespace mx
 
+// Which scale fetch (SCALES_*) a problem's K and scale pointers allow.
+static int scale_mode(const DenseArgs &a) {
+    if (a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0) return SCALES_VEC16;
+    if (a.K % 128 == 0 && aligned(a.as, 4) && aligned(a.bs, 4) && a.ldas % 4 == 0 && a.ldbs % 4 == 0) return SCALES_DWORD;
+    return SCALES_BYTES;
+}
+
 // MX_GEMM_SPLIT=0 in the environment keeps every tile whole (for A/B timing and debugging).
 static bool split_mode() {
     static const bool on = [] {
@@ -391,7 +399,7 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
     a.tiles_n = (a.N + S::BN - 1) / S::BN;
     const int esz = CDT == MX_FP32 ? 4 : 2;
     a.c_vec = aligned(a.c, 16) && (a.ldc * esz) % 16 == 0;
-    const bool k512 = a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0;
+    const int mode = scale_mode(a);
     const int64_t work = (int64_t)a.tiles_m * a.tiles_n * a.split_k;
     const int cus = num_cus();
     a.dp_tiles = (int)work, a.sk_tiles = 0, a.sk_q = 0, a.sk_ws = nullptr;
@@ -402,7 +410,7 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
     // stages, a multiple of 4 (scale fetches are 16-byte aligned) and at least an eighth of a
     // tile, so no tile is cut into more than 9 pieces.
     const int rest = (int)(work % cus);
-    const int KT = a.K >> 7, KT4 = (KT + 3) & ~3;
+    const int KT = ((a.K + 127) >> 7), KT4 = (KT + 3) & ~3;
     if (split_mode() && a.split_k == 1 && !a.accumulate && rest > 0 && KT4 >= 8) {
         int64_t q = ((int64_t)rest * KT4 + cus - 1) / cus;
         if (q < KT4 / 8) q = KT4 / 8;
@@ -418,7 +426,9 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
         }
     }
     dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
-    auto kern = k512 ? gemm_nt_kernel<S, CDT, true> : gemm_nt_kernel<S, CDT, false>;
+    auto kern = mode == SCALES_VEC16   ? gemm_nt_kernel<S, CDT, SCALES_VEC16>
+                : mode == SCALES_DWORD ? gemm_nt_kernel<S, CDT, SCALES_DWORD>
+                                       : gemm_nt_kernel<S, CDT, SCALES_BYTES>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     if (a.sk_tiles)
@@ -427,12 +437,11 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
 }
 
 // 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
-typedef GemmShape<256, 256, 4, 2, true> DenseShape;
+typedef GemmShape<256, 256, 4, 2> DenseShape;
 
 static bool tiled_ok(const DenseArgs &a) {
     const int64_t M = a.M, N = a.N;
-    return a.K % 128 == 0 && aligned(a.aq, 16) && aligned(a.bq, 16) && a.lda % 16 == 0 && a.ldb % 16 == 0 &&
-           aligned(a.as, 4) && aligned(a.bs, 4) && a.ldas % 4 == 0 && a.ldbs % 4 == 0 &&
+    return a.K % MX_BLOCK == 0 && aligned(a.aq, 16) && aligned(a.bq, 16) && a.lda % 16 == 0 && a.ldb % 16 == 0 &&
            256 * a.lda < (int64_t)0x7FFFFFFF && 256 * a.ldb < (int64_t)0x7FFFFFFF &&
            ((M + 255) / 256) * ((N + 255) / 256) * a.split_k < 0x7FFFFFFF;
 }
@@ -468,7 +477,7 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     DenseBatchArgs b;
     int64_t tiles[MX_BATCH_MAX], alone = 0;
     int KT[MX_BATCH_MAX];
-    bool k512 = true;
+    int mode = SCALES_VEC16;  // the least capable fetch any problem needs serves them all
     for (int j = 0; j < count && fuse; j++) {
         DenseArgs &a = probs[j];
         if (!tiled_ok(a)) {
@@ -479,9 +488,9 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         a.tiles_n = (a.N + S::BN - 1) / S::BN;
         a.c_vec = aligned(a.c, 16) && (a.ldc * (CDT == MX_FP32 ? 4 : 2)) % 16 == 0;
         a.dp_tiles = a.tiles_m * a.tiles_n, a.sk_tiles = 0, a.sk_q = 0, a.sk_ws = nullptr;
-        k512 = k512 && a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0;
+        mode = scale_mode(a) > mode ? scale_mode(a) : mode;
         tiles[j] = a.dp_tiles;
-        KT[j] = a.K >> 7;
+        KT[j] = ((a.K + 127) >> 7);
         alone += (tiles[j] + cus - 1) / cus * (KT[j] + 4);
     }
     int share[MX_BATCH_MAX], slices[MX_BATCH_MAX], best_share[MX_BATCH_MAX], best_slices[MX_BATCH_MAX];
@@ -553,7 +562,9 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         b.prob[j] = a;
     }
     b.count = count;
-    auto kern = k512 ? gemm_nt_batch_kernel<S, CDT, true> : gemm_nt_batch_kernel<S, CDT, false>;
+    auto kern = mode == SCALES_VEC16   ? gemm_nt_batch_kernel<S, CDT, SCALES_VEC16>
+                : mode == SCALES_DWORD ? gemm_nt_batch_kernel<S, CDT, SCALES_DWORD>
+                                       : gemm_nt_batch_kernel<S, CDT, SCALES_BYTES>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<dim3((unsigned)b.cu_lo[count]), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
     for (int j = 0; j < count; j++)

@@ -22,12 +22,15 @@
 //   * scales are fetched once per 512 of K (16 bytes per row), byte-transposed 4x4 and
 //     parked in LDS so a lane reads ONE dword per sub-tile per 4 stages and the stage picks
 //     its byte with the instruction's op_sel: no VALU work on scales in the main loop;
-//   * the MFMA is issued "B rows x A rows", so a lane's 4 accumulator registers are 4
-//     consecutive N of one output row; the B rows feeding sub-tiles 4j..4j+3 are permuted so
-//     that sub-tiles (4j, 4j+1) give a lane 8 consecutive N and the four lanes sharing an
-//     output row cover 32 consecutive N between them (sub-tiles (4j+2, 4j+3): the next 32).
-//     One 16-byte store per lane then writes 64 contiguous bytes per output row; a layout
-//     that leaves gaps between the lanes' pieces is issue-bound at ~16 B/clk.
+//   * the MFMA is issued "A rows x B rows": a lane owns 4 consecutive rows (m = 4 (lane / 16) + v)
+//     at one N per sub-tile (n = lane % 16), and the B tile is gathered so that LDS row 16 j + r
+//     of a wave's slice holds B row NT r + j, which makes the NT = 8 sub-tiles of a lane 8
+//     consecutive N: one 16-byte store, and 16 neighbouring lanes write 256 contiguous bytes of
+//     one output row.  The CU's store path coalesces neighbouring lanes only: measured 65-74
+//     B/clk per CU for this layout against 20 B/clk for one that puts neighbouring lanes on
+//     different rows;
+//   * A is held in registers for the stage (MT fragments), B streams through two fragment
+//     buffers, the read of sub-tile j+1 in flight under the MFMAs of sub-tile j.
 #pragma once
 
 #include "mx_common.h"
@@ -62,21 +65,9 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     return (const uint8_t *)(((uint64_t)hi << 32) | lo);
 }
 
-// LANES_N selects how an accumulator tile is spread over the wave:
-//   false  MFMA(B rows, A rows): a lane owns one output row (m = lane % 16) and 4 consecutive N
-//          per sub-tile; B rows are permuted in LDS so two sub-tiles give a lane 8 consecutive N.
-//          Lanes that are neighbours in the wave are neighbours in M, so a store instruction
-//          writes 16 separate 64-byte pieces.
-//   true   MFMA(A rows, B rows): a lane owns 4 consecutive rows (m = 4 (lane / 16) + v) at one N
-//          per sub-tile (n = lane % 16); the B tile is gathered so that LDS row 16 j + r of a
-//          wave's slice holds B row NT r + j, which makes the NT sub-tiles of a lane NT consecutive
-//          N.  16 neighbouring lanes then write 16 x 2 NT contiguous bytes of one output row.
-//          The store path coalesces neighbouring lanes only: measured 65-74 B/clk per CU for this
-//          layout against 20 B/clk for the other.
-template <int BM_, int BN_, int WGM_, int WGN_, bool LANES_N_ = false>
+template <int BM_, int BN_, int WGM_, int WGN_>
 struct GemmShape {
     static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
-    static constexpr bool LANES_N = LANES_N_;
     static constexpr int BK = 128;
     static constexpr int NW = WGM * WGN;
     static constexpr int NTHR = NW * 64;
@@ -86,20 +77,18 @@ struct GemmShape {
     static constexpr int DATA_A = BM * BK, DATA_B = BN * BK;  // bytes per stage
     // Scale planes [buffer][g][row] of dwords; the plane pitch is padded so the 64 lanes of
     // a wave (16 rows x 4 planes) read 64 different banks.
-    static constexpr int PA = BM + 16, PB = LANES_N ? BN + 16 : BN + 32;
+    static constexpr int PA = BM + 16, PB = BN + 16;
     static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
     static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B);
     static constexpr bool TWO_ROWS = BM + BN > NTHR;
-    static_assert(LANES_N || WTN % 64 == 0, "a wave's N extent must be a multiple of 64");
-    static_assert(!LANES_N || NT == 8, "8 sub-tiles along N give a lane 8 consecutive N: one 16-byte store");
+    static_assert(NT == 8, "8 sub-tiles along N give a lane 8 consecutive N: one 16-byte store");
     static_assert(WTM % 16 == 0, "a wave's M extent must be a multiple of 16");
     static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "DMA rows must divide over the waves");
     static_assert(BM + BN <= 2 * NTHR, "scale loader assumes at most two rows per thread");
 };
 
-// chunk swizzles: position of logical 16-byte chunk c of LDS row r is c ^ swz(r)
+// chunk swizzle: position of logical 16-byte chunk c of LDS row r (A or B tile) is c ^ swz_a(r)
 __device__ __forceinline__ int swz_a(int r) { return (r >> 1) & 7; }
-__device__ __forceinline__ int swz_b(int r) { return (((r >> 3) & 3) << 1) | ((r >> 1) & 1); }
 
 // 4x4 byte transpose: in d[s] = bytes {4s+0..4s+3}; out t[g] = bytes {g, 4+g, 8+g, 12+g}.
 __device__ __forceinline__ void transpose4x4(const uint32_t (&d)[4], uint32_t (&t)[4]) {
@@ -132,21 +121,9 @@ __device__ __forceinline__ Lane lane_of() {
     return L;
 }
 
-// Offset, inside a wave's 64-row slice of the B tile, of the rows feeding sub-tile j.
-__device__ __forceinline__ constexpr int b_sub_off(int j) { return (j >> 2) * 64 + ((j & 3) >> 1) * 32 + (j & 1) * 4; }
-
-// Row of the B tile (0..BN-1) that feeds accumulator sub-tile j, MFMA row rr (0..15), for a
-// wave at column wn.  Output column of accumulator register v of lane group g, sub-tile j:
-// wn*WTN + b_sub_off(j) + 8 g + v.
-template <typename S>
-__device__ __forceinline__ int b_tile_row(int wn, int j, int rr) {
-    return wn * S::WTN + b_sub_off(j) + 8 * (rr >> 2) + (rr & 3);
-}
-
 // B row (0..BN-1, relative to the tile) kept in LDS row `r` of the B tile.
 template <typename S>
 __device__ __forceinline__ int b_row_of_lds(int r) {
-    if (!S::LANES_N) return r;  // the permutation lives in the MFMA read offsets (b_tile_row)
     const int in = r % S::WTN;
     return r - in + (in % 16) * S::NT + in / 16;
 }
@@ -160,7 +137,21 @@ struct IssueCtx {
     uint32_t a_voff[S::QA], b_voff[S::QB];
     const uint8_t *srow0, *srow1;  // scale rows tid and tid + NTHR of the [A rows; B rows] list
     int kt0, kt1;                  // K range in 128-byte stages (absolute)
+    // K % 128 != 0: stage tail_kt holds only tail_bytes of K.  Its copies re-read the stage's first
+    // chunk in place of chunks past the end of the row (never past the matrix), and those
+    // chunks' MX blocks carry scale byte 0, so they add nothing.  tail_kt = -1: no such stage.
+    int tail_kt, tail_bytes;
 };
+
+// Byte offset correction of a copy's lane for stage `kt`: 0, or minus the lane's chunk offset when
+// that chunk lies past the end of K.
+template <typename S>
+__device__ __forceinline__ uint32_t tail_fix(const IssueCtx<S> &c, const Lane &L, int kt, int q) {
+    if (kt != c.tail_kt) return 0;
+    const int row = (q * S::NW + L.wave) * 8 + (L.lane >> 3);
+    const int chunk = (L.lane & 7) ^ ((row >> 1) & 7);
+    return chunk * 16 >= c.tail_bytes ? (uint32_t)(chunk * 16) : 0u;
+}
 
 // Row r (0..BM-1) of the A tile and row r of the B tile as the DMA engine sees them.
 template <typename S>
@@ -185,21 +176,35 @@ __device__ __forceinline__ void issue_stage(const IssueCtx<S> &c, const Lane &L,
     const uint32_t la = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf * S::DATA_A + L.wave * 1024);
     const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf * S::DATA_B + L.wave * 1024);
 #pragma unroll
-    for (int q = 0; q < S::QA; q++) dma16(ga, c.a_voff[q], la + q * S::NW * 1024);
+    for (int q = 0; q < S::QA; q++) dma16(ga, c.a_voff[q] - tail_fix<S>(c, L, kt, q), la + q * S::NW * 1024);
 #pragma unroll
-    for (int q = 0; q < S::QB; q++) dma16(gb, c.b_voff[q], lb + q * S::NW * 1024);
+    for (int q = 0; q < S::QB; q++) dma16(gb, c.b_voff[q] - tail_fix<S>(c, L, kt, q), lb + q * S::NW * 1024);
 }
 
+// How a row's scale bytes are fetched: one 16-byte load per 512 of K (K % 512 == 0, 16-byte
+// aligned rows), one dword per stage (K % 128 == 0, 4-byte aligned rows), or byte by byte (any
+// K % 32 == 0 and any pitch; blocks past the end of K read as scale byte 0).
+enum { SCALES_VEC16 = 0, SCALES_DWORD = 1, SCALES_BYTES = 2 };
+
 // 16 scale bytes (4 stages x 4 blocks) of one row starting at scale column kb0.
-template <bool K512>
+template <int MODE>
 __device__ __forceinline__ void load_scales(const uint8_t *row, int kb0, int kb_end, uint32_t (&d)[4]) {
     const uint8_t *p = row + kb0;
-    if (K512) {
+    if (MODE == SCALES_VEC16) {
         v4i t = *(const v4i *)p;
         d[0] = t[0], d[1] = t[1], d[2] = t[2], d[3] = t[3];
-    } else {
+    } else if (MODE == SCALES_DWORD) {
 #pragma unroll
         for (int s = 0; s < 4; s++) d[s] = kb0 + 4 * s < kb_end ? *(const uint32_t *)(p + 4 * s) : 0u;
+    } else {
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                if (kb0 + 4 * s + b < kb_end) w |= (uint32_t)p[4 * s + b] << (8 * b);
+            d[s] = w;
+        }
     }
 }
 
@@ -238,89 +243,45 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
     const uint32_t wa = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf_next * S::DATA_A + L.wave * 1024);
     const uint32_t wb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf_next * S::DATA_B + L.wave * 1024);
     constexpr int NQ = S::QA + S::QB;                      // copies this wave issues per stage
-    constexpr int ISSUE_STEPS = S::MT / 2 > 0 ? S::MT / 2 : 1;  // ... during the first half of the stage
     auto issue = [&](int q) {
-        if (q < S::QA) dma16(ga, c.a_voff[q], wa + q * S::NW * 1024);
-        else dma16(gb, c.b_voff[q - S::QA], wb + (q - S::QA) * S::NW * 1024);
+        if (q < S::QA) dma16(ga, c.a_voff[q] - tail_fix<S>(c, L, kt_next, q), wa + q * S::NW * 1024);
+        else dma16(gb, c.b_voff[q - S::QA] - tail_fix<S>(c, L, kt_next, q - S::QA), wb + (q - S::QA) * S::NW * 1024);
     };
 
-    if constexpr (S::LANES_N) {
-        // A is held (MT fragments), B streams through two fragment buffers.
-        constexpr int STEPS = S::NT / 2 > 0 ? S::NT / 2 : 1;
-        __builtin_amdgcn_sched_barrier(0);
-        v8i bfr[2];
-        {
-            v4i lo = *(const v4i *)(lb + b_lo);
-            v4i hi = *(const v4i *)(lb + b_hi);
-            bfr[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    // A is held (MT fragments), B streams through two fragment buffers.  Nothing crosses into or
+    // out of the stage body, nor from one step of it into the next (sched_barrier).  LDS reads
+    // return in order, so the first MFMA's operands (B[0], A[0]) are asked for first.
+    constexpr int STEPS = S::NT / 2 > 0 ? S::NT / 2 : 1;  // the copies go out during the first half of the stage
+    __builtin_amdgcn_sched_barrier(0);
+    v8i bfr[2];
+    {
+        v4i lo = *(const v4i *)(lb + b_lo);
+        v4i hi = *(const v4i *)(lb + b_hi);
+        bfr[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    v8i afr[S::MT];
+#pragma unroll
+    for (int i = 0; i < S::MT; i++) {
+        v4i lo = *(const v4i *)(la + a_lo + i * (16 * 128));
+        v4i hi = *(const v4i *)(la + a_hi + i * (16 * 128));
+        afr[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < S::NT; j++) {
+        if (j + 1 < S::NT) {
+            v4i lo = *(const v4i *)(lb + b_lo + (j + 1) * (16 * 128));
+            v4i hi = *(const v4i *)(lb + b_hi + (j + 1) * (16 * 128));
+            bfr[(j + 1) & 1] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-        v8i afr[S::MT];
+        if (j < STEPS) {
 #pragma unroll
-        for (int i = 0; i < S::MT; i++) {
-            v4i lo = *(const v4i *)(la + a_lo + i * (16 * 128));
-            v4i hi = *(const v4i *)(la + a_hi + i * (16 * 128));
-            afr[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < S::NT; j++) {
-            if (j + 1 < S::NT) {
-                v4i lo = *(const v4i *)(lb + b_lo + (j + 1) * (16 * 128));
-                v4i hi = *(const v4i *)(lb + b_hi + (j + 1) * (16 * 128));
-                bfr[(j + 1) & 1] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-            if (j < STEPS) {
-#pragma unroll
-                for (int q = j * NQ / STEPS; q < (j + 1) * NQ / STEPS; q++) issue(q);
-            }
-#pragma unroll
-            for (int i = 0; i < S::MT; i++)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(afr[i], bfr[j & 1], acc[i][j], 0, 0, OPSEL,
-                                                                             sa[i], OPSEL, sb[j]);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int q = j * NQ / STEPS; q < (j + 1) * NQ / STEPS; q++) issue(q);
         }
 #pragma unroll
         for (int i = 0; i < S::MT; i++)
-#pragma unroll
-            for (int j = 0; j < S::NT; j++) asm volatile("" : "+v"(acc[i][j]));
-        return;
-    }
-
-    // Nothing crosses into or out of the stage body, nor from one step of it into the next.
-    __builtin_amdgcn_sched_barrier(0);
-    // A fragments are double buffered in registers: the reads for sub-tile i+1 are in
-    // flight while the MFMAs of sub-tile i issue.  LDS reads return in order, so the first
-    // MFMA's operands (A[0], B[0]) are asked for first: it can issue while B[1..] still stream in.
-    v8i af[2];
-    {
-        v4i lo = *(const v4i *)(la + a_lo);
-        v4i hi = *(const v4i *)(la + a_hi);
-        af[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-    v8i bf[S::NT];
-#pragma unroll
-    for (int j = 0; j < S::NT; j++) {
-        const int o = b_sub_off(j) * 128;
-        v4i lo = *(const v4i *)(lb + b_lo + o);
-        v4i hi = *(const v4i *)(lb + b_hi + o);
-        bf[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < S::MT; i++) {
-        if (i + 1 < S::MT) {
-            v4i lo = *(const v4i *)(la + a_lo + (i + 1) * (16 * 128));
-            v4i hi = *(const v4i *)(la + a_hi + (i + 1) * (16 * 128));
-            af[(i + 1) & 1] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-        if (i < ISSUE_STEPS) {
-#pragma unroll
-            for (int q = i * NQ / ISSUE_STEPS; q < (i + 1) * NQ / ISSUE_STEPS; q++) issue(q);
-        }
-#pragma unroll
-        for (int j = 0; j < S::NT; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i & 1], acc[i][j], 0, 0, OPSEL,
-                                                                         sb[j], OPSEL, sa[i]);
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(afr[i], bfr[j & 1], acc[i][j], 0, 0, OPSEL, sa[i],
+                                                                         OPSEL, sb[j]);
         __builtin_amdgcn_sched_barrier(0);
     }
     // The MFMAs have no side effects the compiler can see, so it would sink them past the
@@ -365,7 +326,7 @@ struct LdsScratch {
 //                                           lane issued if that number is the same compile-time
 //                                           constant P::NST for the whole wave, else -1
 //   int  P::kb_end                          scale bytes per row (bound for predicated fetches)
-template <typename S, bool K512, typename P>
+template <typename S, int K512, typename P>  // K512: one of SCALES_*
 __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     uint8_t *const ldsA = smem;                                                  // [2][BM*128]
     uint8_t *const ldsB = smem + 2 * S::DATA_A;                                  // [2][BN*128]
@@ -378,9 +339,9 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
 
     // per-lane LDS read offsets: low half = 16-byte chunk g, high half = chunk g + 4 (= offset ^ 64)
     const int a_row = L.wm * S::WTM + L.r16;
-    const int b_row = S::LANES_N ? L.wn * S::WTN + L.r16 : b_tile_row<S>(L.wn, 0, L.r16);
+    const int b_row = L.wn * S::WTN + L.r16;
     const int a_rd = a_row * 128 + ((L.g ^ swz_a(a_row)) << 4);
-    const int b_rd = b_row * 128 + ((L.g ^ (S::LANES_N ? swz_a(b_row) : swz_b(b_row))) << 4);
+    const int b_rd = b_row * 128 + ((L.g ^ swz_a(b_row)) << 4);
 
     typename P::Tile cur, nxt;
     if (!prob.next(cur)) return;
@@ -420,7 +381,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             for (int i = 0; i < S::MT; i++) sa[i] = (int)ldsSA[(sbuf * 4 + L.g) * S::PA + a_row + 16 * i];
 #pragma unroll
             for (int j = 0; j < S::NT; j++)
-                sb[j] = (int)ldsSB[(sbuf * 4 + L.g) * S::PB + b_row + (S::LANES_N ? 16 * j : b_sub_off(j))];
+                sb[j] = (int)ldsSB[(sbuf * 4 + L.g) * S::PB + b_row + 16 * j];
 
             // One K stage.  In every stage but the tile's last, the next stage's operands are
             // put in flight during the stage and waited for at its end.

@@ -141,12 +141,11 @@ struct GroupedProblem {
     // scan_pad 128-row tiles of the padded token axis
     int scan_e, scan_tiles, scan_pad;
 
-    // Accumulator layout (GemmShape LANES_N): lane (r16, g) holds, for sub-tile (i, j) and
+    // Accumulator layout: lane (r16, g) holds, for sub-tile (i, j) and
     // register v, row 16 i + 4 g + v of the wave's 64 rows and column 8 r16 + j of its 128.
     // GEMM1 fills each wave's 128-row slice of the B tile with 64 gate rows (sub-tiles 0-3) and
     // the 64 value rows of the same hidden units (sub-tiles 4-7), so a tile spans BN/2 hidden
     // units and a lane owns 4 consecutive ones, gate and value.
-    static_assert(S::LANES_N, "the expert kernels use the layout that puts neighbouring lanes on neighbouring N");
     static constexpr int N_PER_TILE = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
@@ -224,6 +223,7 @@ struct GroupedProblem {
         c.b_base = p.wq + (int64_t)t.expert * p.stride_we;
         c.kt0 = t.kt0;
         c.kt1 = t.kt1;
+        c.tail_kt = -1, c.tail_bytes = 0;  // K % 128 == 0 is a precondition of these kernels
 #pragma unroll
         for (int q = 0; q < S::QA; q++) {
             const int row = dma_row<S>(L, q);
@@ -537,7 +537,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t *__restrict
     *(v4i *)(out + t * ldo + c) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
 }
 
-template <typename S, int MODE, int CDT, bool K512>
+template <typename S, int MODE, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void grouped_kernel(GroupedArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     GroupedProblem<S, MODE, CDT> prob(args);
@@ -711,6 +711,7 @@ struct WgradProblem {
         c.b_base = p.bq + (int64_t)t.n0 * p.ldb;
         c.kt0 = t.kt0;
         c.kt1 = t.kt1;
+        c.tail_kt = -1, c.tail_bytes = 0;  // K % 128 == 0 is a precondition of these kernels
         const int mrem = p.N - t.m0, nrem = p.Kout - t.n0;
 #pragma unroll
         for (int q = 0; q < S::QA; q++) {
@@ -764,7 +765,7 @@ template <typename S, int CDT>
 __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     WgradProblem<S, CDT> prob(args);
-    persistent_gemm<S, false>(prob, smem);
+    persistent_gemm<S, SCALES_DWORD>(prob, smem);
 }
 
 // Adds the K slices of every tile of every non-empty expert, in slice order, and stores dW.
@@ -818,7 +819,7 @@ using namespace mx;
 static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
 // 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
-typedef GemmShape<256, 256, 4, 2, true> Big;
+typedef GemmShape<256, 256, 4, 2> Big;
 
 static bool tiled_ok(const GroupedArgs &a, int64_t a_rows) {
     return a.K % 128 == 0 && aligned(a.xq, 16) && aligned(a.wq, 16) && a.ldx % 16 == 0 && a.ldw % 16 == 0 &&
@@ -838,7 +839,7 @@ static int launch_grouped(GroupedArgs a, hipStream_t st) {
                       a.ldws % 16 == 0 && a.stride_wse % 16 == 0;
     const int cus = num_cus();
     dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
-    auto kern = k512 ? grouped_kernel<S, MODE, CDT, true> : grouped_kernel<S, MODE, CDT, false>;
+    auto kern = k512 ? grouped_kernel<S, MODE, CDT, SCALES_VEC16> : grouped_kernel<S, MODE, CDT, SCALES_DWORD>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;

@@ -48,8 +48,11 @@ SHAPES = [
     (1, 16, 1024),
     (1000, 72, 256),
     (512, 768, 2048),
-    (64, 64, 96),  # K % 128 != 0: generic kernel
+    (64, 64, 96),  # K % 128 != 0: the last K stage is partial
     (130, 50, 32),
+    (300, 200, 160),
+    (512, 384, 4000),  # 31 full stages + 32 of K; scale rows of 125 bytes: byte-wise scale fetch
+    (1024, 512, 2080),
 ]
 
 
@@ -148,6 +151,7 @@ SPLIT_SHAPES = [
     (256, 256, 16384),  # a single tile
     (2048, 1536, 2048),  # 48 tiles
     (4352, 4096, 1024),  # one whole round of 256 tiles, then 16 more that are split
+    (768, 512, 8160),  # K % 128 == 96: the partial stage ends the last piece of every tile
 ]
 
 
@@ -205,6 +209,20 @@ def test_gemm_batch(oracle, shapes, dtype):
     with pytest.raises(ValueError):
         _mx().mxfp8_matmul_pq_batch([(dev_ops[0][0], dev_ops[0][1], dev_ops[0][2][:, :32], dev_ops[0][3])], dtype)
     assert _mx().mxfp8_matmul_pq_batch([], dtype) == []
+
+
+def test_gemm_unaligned_operands_take_the_generic_kernel(oracle):
+    """Row pitches that are not multiples of 16 bytes cannot feed the copy engine: the slow kernel serves them."""
+    m, n, k = 96, 80, 256
+    aq, as_, bq, bs = _operands(oracle, m, n, k)
+    ref = oracle.gemm_nt(aq, as_, bq, bs)
+    f8 = torch.float8_e4m3fn
+    wide_a = torch.zeros(m, k + 8, dtype=torch.uint8, device=DEV)
+    wide_a[:, :k] = aq.to(DEV)
+    wide_b = torch.zeros(n, k + 24, dtype=torch.uint8, device=DEV)
+    wide_b[:, :k] = bq.to(DEV)
+    got = _mx().mxfp8_matmul_pq(wide_a[:, :k].view(f8), as_.to(DEV), wide_b[:, :k].view(f8), bs.to(DEV), torch.float32)
+    assert oracle.rel_error(got.cpu(), ref) < TOL_FP32
 
 
 def test_gemm_split_k_accumulate(oracle):
