@@ -402,41 +402,61 @@ struct GroupedProblem {
     }
 
     // ---- DGRAD2: the accumulator dout[t] . W_out is consumed three ways in registers
+    // Everything a 16-row slab (one i: the lane's 4 rows) reads from memory -- pair index, gate,
+    // the fp8 copy of h, the stored pre -- is requested before any of it is used: issued row by
+    // row, each dependent chain (order -> gate) and each row's loads would expose a full memory
+    // latency 16 times per tile, which made this epilogue several times longer than the K loop.
     __device__ __forceinline__ int epilogue_dgrad2(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
         const int H = p.N;
         const int hblock = t.n0 + L.wn * S::WTN + 32 * (L.r16 >> 2);  // the 32 hidden units of a quad
         const int h = t.n0 + L.wn * S::WTN + 8 * L.r16;
+        const bool col_ok = hblock < H;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
+            int pair[4];
+            float gate[4];
+            v2i hc[4];
+            uint32_t hsb[4];
+            v4i pg[4], pv[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int m = row_of(t, L, i, v);
+                const int mm = m < t.end ? m : t.end - 1;
+                pair[v] = p.order[mm];
+                const int hh = col_ok ? h : 0, hb = col_ok ? hblock : 0;  // clamped: loaded, never used
+                hc[v] = *(const v2i *)(p.hq + (int64_t)mm * p.ldhq + hh);
+                hsb[v] = p.hs[(int64_t)mm * p.ldhs + (hb >> 5)];
+                const uint16_t *pp = (const uint16_t *)p.pre + (int64_t)mm * p.ldpre + hh;
+                pg[v] = *(const v4i *)pp;
+                pv[v] = *(const v4i *)(pp + H);
+            }
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                gate[v] = p.gate_f32 ? ((const float *)p.gate)[pair[v]] : load_act<CDT>(p.gate, pair[v]);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int m = row_of(t, L, i, v);
                 const bool row_ok = m < t.end;
-                const int mm = row_ok ? m : t.end - 1;
-                const int pair = p.order[mm];
-                const float gate = p.gate_f32 ? ((const float *)p.gate)[pair] : load_act<CDT>(p.gate, pair);
-                const bool ok = row_ok && hblock < H;
+                const bool ok = row_ok && col_ok;
                 float a[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) a[e] = acc[i][e][v];
                 float dg[8], dv[8], dot = 0.0f;
                 if (ok) {
                     // h read back from its fp8 copy: the forward multiplied those values
-                    const v2i hc = *(const v2i *)(p.hq + (int64_t)mm * p.ldhq + h);
-                    const float hscale = bits2f((uint32_t)p.hs[(int64_t)mm * p.ldhs + (hblock >> 5)] << 23);
+                    const float hscale = bits2f(hsb[v] << 23);
                     float gq[8], vq[8];
-                    const uint16_t *pp = (const uint16_t *)p.pre + (int64_t)mm * p.ldpre + h;
-                    unpack8<CDT>(*(const v4i *)pp, gq);
-                    unpack8<CDT>(*(const v4i *)(pp + H), vq);
+                    unpack8<CDT>(pg[v], gq);
+                    unpack8<CDT>(pv[v], vq);
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
                         typedef float v2f __attribute__((ext_vector_type(2)));
-                        const int word = hc[e >> 2];
+                        const int word = hc[v][e >> 2];
                         const v2f pairv = (e & 2) ? __builtin_amdgcn_cvt_pk_f32_fp8(word, true)
                                                   : __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
                         const float hval = pairv[e & 1] * hscale;
                         dot += a[e] * hval;
-                        const float dh = a[e] * gate;
+                        const float dh = a[e] * gate[v];
                         const float sg = sigmoid_f(gq[e]);
                         dg[e] = dh * vq[e] * sg * (1.0f + gq[e] * (1.0f - sg));
                         dv[e] = dh * gq[e] * sg;
@@ -479,7 +499,7 @@ struct GroupedProblem {
                 }
                 // the dot product over the expert width is split across lanes, waves and N tiles
                 dot = row16_sum(dot);
-                if (row_ok && L.r16 == 0) atomicAdd(p.dgate + pair, dot);
+                if (row_ok && L.r16 == 0) atomicAdd(p.dgate + pair[v], dot);
             }
         }
         return -1;
