@@ -257,3 +257,47 @@ def test_gemm_errors():
         mx.mxfp8_matmul_pq(a, s[:, :1], a, s)
     with pytest.raises(ValueError):
         mx.mxfp8_matmul(torch.zeros(4, 48, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 48, dtype=torch.bfloat16, device=DEV))
+
+
+def test_gemm_random_shapes(oracle):
+    """Seeded sweep over ragged M, N and every K % 32 class against the fp64 oracle, single and batched."""
+    import random
+
+    rnd = random.Random(SEED)
+    f8 = torch.float8_e4m3fn
+    problems, refs = [], []
+    for case in range(24):
+        m = rnd.choice([1, 7, 64, 255, 256, 257, 300, 511, 777])
+        n = rnd.choice([8, 16, 72, 200, 256, 264, 520])
+        k = 32 * rnd.randint(1, 40)
+        aq, as_, bq, bs = _operands(oracle, m, n, k, seed=SEED + case)
+        ref = oracle.gemm_nt(aq, as_, bq, bs)
+        dev = (aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV))
+        got = _mx().mxfp8_matmul_pq(*dev, torch.float32)
+        assert oracle.rel_error(got.cpu(), ref) < TOL_FP32, (m, n, k)
+        problems.append(dev)
+        refs.append(ref)
+    outs = _mx().mxfp8_matmul_pq_batch(problems, torch.bfloat16)
+    for out, ref, dev in zip(outs, refs, problems):
+        assert oracle.rel_error(out.cpu(), ref) < TOL_BF16, tuple(dev[0].shape)
+
+
+def test_gemm_split_on_two_streams(oracle):
+    """Launches that use the K-split scratch on different streams at the same time do not share it."""
+    m, n, k = 512, 512, 8192  # 4 tiles, long K: the even split
+    f8 = torch.float8_e4m3fn
+    ops = [_operands(oracle, m, n, k, seed=SEED + i) for i in range(2)]
+    refs = [oracle.gemm_nt(*op) for op in ops]
+    devs = [(aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)) for aq, as_, bq, bs in ops]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    outs = [[], []]
+    for rep in range(8):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                outs[i].append(_mx().mxfp8_matmul_pq(*devs[i], torch.float32))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for out in outs[i]:
+            assert torch.equal(out, outs[i][0])
+        assert oracle.rel_error(outs[i][0].cpu(), refs[i]) < TOL_FP32
