@@ -240,7 +240,11 @@ int mx_experts_combine(const void *y, int64_t ldy, const int32_t *order, const i
  * (M,H); dgate[order[m]] += <acc, dequant(hq,hs)[m]> (fp32 atomics, caller-zeroed);
  * dh = acc * gate[order[m]]; SwiGLU backward from the stored pre; dpre (M,2H) stored in
  * act_dtype and quantized from the fp32 values into dpq (M,2H), dps (M,2H/32).
- * Replaces _experts_gemm2_dgrad (src/kohakuwullm/kernels/mxfp8/experts_bwd.py:29-164).
+ * Optional (both or neither): ptq (2H,Mpad), pts (2H,Mpad/32) receive the stored (rounded)
+ * dpre quantized along the tokens in the padded layout of mx_quantize_cols_grouped, bit for
+ * bit what that quantizer makes of dpre; dpre itself may then be NULL and is not written.
+ * Replaces _experts_gemm2_dgrad (src/kohakuwullm/kernels/mxfp8/experts_bwd.py:29-164); with
+ * ptq it also stands in for the dpre pass of _quantize_cols_grouped (quant.py, WGRAD of GEMM1).
  */
 int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int64_t T, int64_t lddq, int64_t ldds,
                            const int32_t *token_of, const int32_t *order, const void *gate, int gate_dtype,
@@ -248,6 +252,7 @@ int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int64_t T, int6
                            int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
                            const uint8_t *hq, int64_t ldhq, const uint8_t *hs, int64_t ldhs, const void *pre,
                            void *dpre, int64_t ldpre, uint8_t *dpq, int64_t lddpq, uint8_t *dps, int64_t lddps,
+                           uint8_t *ptq, int64_t ldptq, uint8_t *pts, int64_t ldpts,
                            float *dgate, int act_dtype, int64_t M, int64_t H, int64_t K, void *stream);
 
 /*

@@ -44,7 +44,7 @@ SIGNATURES = {
               _i64, _i64, _i64, _p]),
     "mx_experts_gemm2_dgrad": (
         _ci, [_p, _p, _i64, _i64, _i64, _p, _p, _p, _ci, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64,
-              _p, _p, _i64, _p, _i64, _p, _i64, _p, _ci, _i64, _i64, _i64, _p]),
+              _p, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _ci, _i64, _i64, _i64, _p]),
     "mx_experts_combine": (_ci, [_p, _i64, _p, _p, _i64, _p, _ci, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _p]),
     "mx_quantize_cols_grouped": (
         _ci, [_p, _ci, _i64, _i64, _ci, _p, _p, _ci, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _p]),

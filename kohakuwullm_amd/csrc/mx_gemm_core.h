@@ -314,8 +314,9 @@ __device__ __forceinline__ void wait_vm_allow_c() {
 // last K stage was read from.  An epilogue may use them as scratch once every wave has left
 // the main loop (a workgroup barrier of its own first); the buffer is not written again before
 // the barrier that follows the epilogue.
+// `c`: the scale planes of the tile's last super-step (4 * PA words), free under the same rule.
 struct LdsScratch {
-    uint8_t *a, *b;
+    uint8_t *a, *b, *c;
 };
 
 // The persistent tile loop.  `P` (the problem policy) provides
@@ -433,7 +434,8 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         // of stores the wait lets exactly those stay in flight,
         // so the stores drain under the next tile's first stage.
         const int lastbuf = (gstage - 1) & 1;
-        const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B});
+        const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B,
+                                            (uint8_t *)(ldsSA + ((gsuper - 1) & 1) * 4 * S::PA)});
         if (has_next) {
             if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
             if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);

@@ -94,6 +94,13 @@ __device__ __forceinline__ void unpack8(const v4i &w, float (&v)[8]) {
     }
 }
 
+// One 16-bit storage value (in the low half of `bits`) as fp32.
+template <int CDT>
+__device__ __forceinline__ float unpack1(uint32_t bits) {
+    if (CDT == MX_BF16) return bits2f(bits << 16);
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+
 template <int CDT>
 __device__ __forceinline__ void atomic_add2(void *base, int64_t off, float a, float b) {
     if (CDT == MX_BF16) {
@@ -247,7 +254,7 @@ struct GroupedProblem {
         if constexpr (MODE == MODE_PLAIN) return epilogue_plain(t, L, acc);
         else if constexpr (MODE == MODE_GEMM1) return epilogue_gemm1(t, L, acc, lds);
         else if constexpr (MODE == MODE_SCATTER) return epilogue_scatter(t, L, acc);
-        else return epilogue_dgrad2(t, L, acc);
+        else return epilogue_dgrad2(t, L, acc, lds);
     }
 
     // sorted row of (i, v) for this lane
@@ -406,7 +413,19 @@ struct GroupedProblem {
     // the fp8 copy of h, the stored pre -- is requested before any of it is used: issued row by
     // row, each dependent chain (order -> gate) and each row's loads would expose a full memory
     // latency 16 times per tile, which made this epilogue several times longer than the K loop.
-    __device__ __forceinline__ int epilogue_dgrad2(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT]) const {
+    //
+    // Token axis (p.htq given): dpre is also wanted quantized along the tokens, for dW_in.  The
+    // lane keeps its 16 rows x 16 columns of dpre as packed 16-bit values -- the stored, rounded
+    // ones, which is what a column quantizer reading dpre back would see -- in place of the
+    // accumulators they were computed from, and a second phase quantizes them in 32-row blocks and
+    // transposes them through the free stage buffer, 128 columns of dpre at a time.
+    __device__ __forceinline__ int epilogue_dgrad2(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT],
+                                                   const LdsScratch &lds) const {
+        static_assert(S::MT % 2 == 0 && (S::BN / 2) * S::BM <= S::DATA_A && (S::BN / 2) * S::BM <= S::DATA_B &&
+                          2 * (S::BN / 2) * (S::BM / 32) <= 4 * S::PA * 4,
+                      "token-axis staging: 128 columns per pass, two passes in flight");
+        const bool tok = p.htq != nullptr;
+        uint32_t keep[2][S::MT][4][4];  // [gate | value][slab][row][pair of columns]
         const int H = p.N;
         const int hblock = t.n0 + L.wn * S::WTN + 32 * (L.r16 >> 2);  // the 32 hidden units of a quad
         const int h = t.n0 + L.wn * S::WTN + 8 * L.r16;
@@ -480,9 +499,13 @@ struct GroupedProblem {
                         round_pair<CDT>(tg[2 * e], tg[2 * e + 1], w[e]);
                         round_pair<CDT>(tv[2 * e], tv[2 * e + 1], x[e]);
                     }
-                    uint16_t *dp = (uint16_t *)p.dpre + (int64_t)m * p.ldpre + h;
-                    *(v4i *)dp = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-                    *(v4i *)(dp + H) = v4i{(int)x[0], (int)x[1], (int)x[2], (int)x[3]};
+                    if (p.dpre) {
+                        uint16_t *dp = (uint16_t *)p.dpre + (int64_t)m * p.ldpre + h;
+                        *(v4i *)dp = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                        *(v4i *)(dp + H) = v4i{(int)x[0], (int)x[1], (int)x[2], (int)x[3]};
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) keep[0][i][v][e] = w[e], keep[1][i][v][e] = x[e];
                     v2i cg, cv;
                     cg[0] = (int)pack4_e4m3(dg[0] * ig, dg[1] * ig, dg[2] * ig, dg[3] * ig);
                     cg[1] = (int)pack4_e4m3(dg[4] * ig, dg[5] * ig, dg[6] * ig, dg[7] * ig);
@@ -496,10 +519,82 @@ struct GroupedProblem {
                         sp[0] = (uint8_t)bg;
                         sp[H >> 5] = (uint8_t)bv;
                     }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) keep[0][i][v][e] = keep[1][i][v][e] = 0u;  // padding rows and columns
                 }
                 // the dot product over the expert width is split across lanes, waves and N tiles
                 dot = row16_sum(dot);
                 if (row_ok && L.r16 == 0) atomicAdd(p.dgate + pair[v], dot);
+            }
+        }
+        if (!tok) return -1;
+
+        __syncthreads();  // every wave is out of the main loop: the stage buffer is free
+        const int64_t pbase = t.ppos;
+#pragma unroll
+        for (int pass = 0; pass < 4; pass++) {
+            // pass = (gate | value, low | high four of the lane's eight columns); staged column
+            // c = 64 wn + 4 r16 + e holds tile column 8 (c / 4) + 4 sub + c % 4
+            // The passes alternate between the two halves of the stage buffer (and of the scale
+            // area), so one barrier per pass is enough: a half is rewritten two passes later, with
+            // the next pass's barrier in between, and a pass's global stores drain under the
+            // arithmetic of the next.
+            const int half = pass >> 1, sub = pass & 1;
+            uint8_t *const codes = (pass & 1) ? lds.b : lds.a;
+            uint8_t *const bytes = lds.c + (pass & 1) * ((S::BN / 2) * (S::BM / 32));
+#pragma unroll
+            for (int blk = 0; blk < S::MT / 2; blk++) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float val[2][4];
+                    float cm = 0.0f;
+#pragma unroll
+                    for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            const uint32_t word = keep[half][2 * blk + ii][v][2 * sub + (e >> 1)];
+                            val[ii][v] = unpack1<CDT>((e & 1) ? word >> 16 : word & 0xFFFFu);
+                            cm = fmaxf(cm, fabsf(val[ii][v]));
+                        }
+                    // the block's 32 rows are this lane's 8 values and the lanes 16, 32, 48 away
+                    cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+                    cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+                    const uint32_t byte = scale_byte(cm);
+                    const float inv = inv_scale(byte);
+                    const int col = L.wn * (S::WTN / 2) + 4 * L.r16 + e;
+#pragma unroll
+                    for (int ii = 0; ii < 2; ii++) {
+                        const int row = L.wm * S::WTM + 16 * (2 * blk + ii) + 4 * L.g;  // 4 consecutive rows: one dword
+                        const uint32_t w = pack4_e4m3(val[ii][0] * inv, val[ii][1] * inv, val[ii][2] * inv, val[ii][3] * inv);
+                        // column-major, 256 bytes per column, 16-byte chunks XOR-swizzled by the lane's r16
+                        *(uint32_t *)(codes + col * S::BM + ((((row >> 4) ^ (col >> 2)) & 15) << 4) + (row & 15)) = w;
+                    }
+                    if (L.g == 0) bytes[col * (S::BM / 32) + L.wm * (S::WTM / 32) + blk] = (uint8_t)byte;
+                }
+            }
+            __syncthreads();
+            // 16 consecutive lanes write the 256 bytes of one column's 256 tokens; a 128-row half
+            // that starts past the expert's rows belongs to the next expert's padding and is skipped
+#pragma unroll
+            for (int k = 0; k < (S::BN / 2) * S::BM / 16 / S::NTHR; k++) {
+                const int q = L.tid + k * S::NTHR;
+                const int col = q >> 4, ch = q & 15;
+                const int hcol = t.n0 + 8 * (col >> 2) + 4 * sub + (col & 3);
+                const bool half_ok = t.row0 + (ch >> 3) * 128 < t.end;
+                if (hcol < H && half_ok) {
+                    const v4i w = *(const v4i *)(codes + col * S::BM + (((ch ^ (col >> 2)) & 15) << 4));
+                    *(v4i *)(p.htq + (int64_t)(half * H + hcol) * p.ldhtq + pbase + ch * 16) = w;
+                }
+            }
+            if (L.tid < S::BN / 2) {
+                const int hcol = t.n0 + 8 * (L.tid >> 2) + 4 * sub + (L.tid & 3);
+                if (hcol < H) {
+                    const uint32_t *src = (const uint32_t *)(bytes + L.tid * (S::BM / 32));
+                    uint8_t *dst = p.hts + (int64_t)(half * H + hcol) * p.ldhts + (pbase >> 5);
+                    *(uint32_t *)dst = src[0];
+                    if (t.row0 + 128 < t.end) *(uint32_t *)(dst + 4) = src[1];
+                }
             }
         }
         return -1;
@@ -963,20 +1058,25 @@ extern "C" int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int6
                                       int64_t stride_wse, int64_t ldws, const int32_t *offsets, int64_t E,
                                       const uint8_t *hq, int64_t ldhq, const uint8_t *hs, int64_t ldhs, const void *pre,
                                       void *dpre, int64_t ldpre, uint8_t *dpq, int64_t lddpq, uint8_t *dps,
-                                      int64_t lddps, float *dgate, int act_dtype, int64_t M, int64_t H, int64_t K,
-                                      void *stream) {
+                                      int64_t lddps, uint8_t *ptq, int64_t ldptq, uint8_t *pts, int64_t ldpts,
+                                      float *dgate, int act_dtype, int64_t M, int64_t H, int64_t K, void *stream) {
     if (!sizes_ok(E, M, H, K) || H % MX_BLOCK || lddq < K || ldw < K || ldhq < H || ldpre < 2 * H || lddpq < 2 * H ||
-        lddps < 2 * H / MX_BLOCK || !token_of || !order || !gate || !pre || !dpre || !dgate)
+        lddps < 2 * H / MX_BLOCK || !token_of || !order || !gate || !pre || !dgate || (!dpre && !ptq) ||
+        (ptq != nullptr) != (pts != nullptr))
         return MX_EINVAL;
     if (gate_dtype != MX_FP32 && gate_dtype != act_dtype) return MX_EINVAL;
+    const int64_t mpad = ((M + 127) / 128 + E) * 128;
+    if (ptq && (ldptq < mpad - 128 * E || ldpts < (mpad - 128 * E) / MX_BLOCK)) return MX_EINVAL;
     if (M == 0 || H == 0) return MX_OK;
     GroupedArgs a = base_args(dq, ds, lddq, ldds, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
     a.token_of = token_of, a.order = order, a.gate = gate, a.gate_f32 = gate_dtype == MX_FP32;
     a.hq = (uint8_t *)hq, a.ldhq = ldhq, a.hs = (uint8_t *)hs, a.ldhs = ldhs;
     a.pre = (void *)pre, a.dpre = dpre, a.ldpre = ldpre, a.dpq = dpq, a.lddpq = lddpq, a.dps = dps, a.lddps = lddps;
     a.dgate = dgate;
-    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || !aligned(pre, 16) || !aligned(dpre, 16) ||
-        ldpre % 8 || H % 8 || !aligned(dpq, 8) || lddpq % 8)
+    a.htq = ptq, a.ldhtq = ldptq, a.hts = pts, a.ldhts = ldpts;
+    if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || !aligned(pre, 16) || (dpre && !aligned(dpre, 16)) ||
+        ldpre % 8 || H % 8 || !aligned(dpq, 8) || lddpq % 8 ||
+        (ptq && (!aligned(ptq, 16) || ldptq % 16 || !aligned(pts, 4) || ldpts % 4)))
         return MX_EUNSUPPORTED;
     return launch_grouped_dt<MODE_DGRAD2>(act_dtype, a, (hipStream_t)stream);
 }

@@ -139,16 +139,25 @@ def _routed_product(aq, a_s, wq, ws, token_of, order, gate, offsets, tokens: int
     return out
 
 
-def launch_gemm2_dgrad(dq, ds, token_of, order, gate, wq, ws, hq, hs, pre, dpre, dpq, dps, dgate, offsets) -> None:
+def launch_gemm2_dgrad(dq, ds, token_of, order, gate, wq, ws, hq, hs, pre, dpre, dpq, dps, dgate, offsets,
+                       ptq=None, pts=None) -> None:
+    """DGRAD through GEMM2 with its epilogue.
+
+    ``ptq``/``pts`` ``(2H, Mpad)``/``(2H, Mpad//32)``, when given, receive ``dpre`` quantized along the
+    tokens; ``dpre`` may then be ``None``.
+    """
     m = token_of.numel()
     hidden, dim = wq.shape[1], wq.shape[2]
     _lib.invoke(
         "mx_experts_gemm2_dgrad", 2.0 * m * hidden * dim, dq,
         dq.data_ptr(), ds.data_ptr(), dq.shape[0], dq.stride(0), ds.stride(0), token_of.data_ptr(), order.data_ptr(),
         gate.data_ptr(), _lib.MX_DTYPE[gate.dtype], *_w_args(wq, ws), offsets.data_ptr(), wq.shape[0],
-        hq.data_ptr(), hq.stride(0), hs.data_ptr(), hs.stride(0), pre.data_ptr(), dpre.data_ptr(), pre.stride(0),
-        dpq.data_ptr(), dpq.stride(0), dps.data_ptr(), dps.stride(0), dgate.data_ptr(), _lib.MX_DTYPE[pre.dtype],
-        m, hidden, dim,
+        hq.data_ptr(), hq.stride(0), hs.data_ptr(), hs.stride(0), pre.data_ptr(),
+        0 if dpre is None else dpre.data_ptr(), pre.stride(0),
+        dpq.data_ptr(), dpq.stride(0), dps.data_ptr(), dps.stride(0),
+        0 if ptq is None else ptq.data_ptr(), 0 if ptq is None else ptq.stride(0),
+        0 if pts is None else pts.data_ptr(), 0 if pts is None else pts.stride(0),
+        dgate.data_ptr(), _lib.MX_DTYPE[pre.dtype], m, hidden, dim,
     )
 
 
@@ -188,12 +197,19 @@ class _MXFP8Experts(torch.autograd.Function):
         dev = dout.device
         dout = dout.contiguous()
         dq, ds = quantize_mx(dout)
-        dpre = torch.empty(m, 2 * hidden, device=dev, dtype=dout.dtype)
         dpq = torch.empty(m, 2 * hidden, device=dev, dtype=_FP8)
         dps = torch.empty(m, 2 * hidden // BLOCK_SCALE, device=dev, dtype=torch.uint8)
         # fp32 and zeroed: this reduction crosses workgroups through an atomic
         dgate = torch.zeros(gate.numel(), device=dev, dtype=torch.float32)
-        launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets)
+        ptq = pts = None
+        if ctx.needs_input_grad[1]:
+            # dpre along the tokens, for dW_in: written by the epilogue; dpre itself never reaches memory
+            mpad = padded_rows(m, packed.in_fwd[0].shape[0])
+            ptq = torch.empty(2 * hidden, mpad, device=dev, dtype=_FP8)
+            pts = torch.empty(2 * hidden, mpad // BLOCK_SCALE, device=dev, dtype=torch.uint8)
+        dpre = None if ptq is not None else torch.empty(m, 2 * hidden, device=dev, dtype=dout.dtype)
+        launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets,
+                           ptq, pts)
         dx = _routed_product(dpq, dps, *packed.in_dgrad, token_of, order, None, offsets, rows, top_k, dout.dtype)
 
         dw_in = dw_out = None
@@ -203,7 +219,6 @@ class _MXFP8Experts(torch.autograd.Function):
             dw_out = grouped_mxfp8_wgrad(dtq, dts, htq, hts, offsets, m, dout.dtype)
         if ctx.needs_input_grad[1]:
             # dW_in[e] = dpre rows of e .T @ x rows of e
-            ptq, pts = quantize_mx_cols_grouped(dpre, offsets, m)
             xtq, xts = quantize_mx_cols_grouped(x, offsets, m, index=token_of)
             dw_in = grouped_mxfp8_wgrad(ptq, pts, xtq, xts, offsets, m, dout.dtype)
         return dx, dw_in, dw_out, dgate.to(gate.dtype), None, None, None, None, None

@@ -337,6 +337,67 @@ def test_gemm1_intermediates(oracle):
     assert (hs.cpu() != ref["hs"]).float().mean() < 0.02
 
 
+def test_gemm2_dgrad_token_axis(oracle):
+    """The dgrad epilogue's token-axis copy of dpre is the grouped column quantizer's result on the stored dpre, bit for
+    bit, and asking for it changes none of the other outputs (dpre itself becomes optional)."""
+    from kohakuwullm_amd.kernels.mxfp8.grouped import padded_rows, quantize_mx_cols_grouped
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, launch_gemm1, launch_gemm2_dgrad
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator().manual_seed(SEED + 7)
+    for counts, hid in (([200, 0, 56, 300], 160), ([256, 256], 256), ([1, 700], 544)):
+        top_k = 1
+        e, dim = len(counts), 128
+        tokens = sum(counts)
+        offsets, order, token_of = _routing(counts, top_k, tokens)
+        x = torch.randn(tokens, dim, generator=g).bfloat16()
+        w_in = (torch.randn(e, 2 * hid, dim, generator=g) * 0.08).bfloat16()
+        w_out = (torch.randn(e, dim, hid, generator=g) * 0.08).bfloat16()
+        gate = (torch.rand(tokens, generator=g) * 0.5 + 0.5).bfloat16().to(DEV)
+        dout = torch.randn(tokens, dim, generator=g).bfloat16().to(DEV)
+        packed = MXFP8ExpertWeights(w_in.to(DEV), w_out.to(DEV))
+        m = sum(counts)
+        off_d, tok_d, ord_d = offsets.to(DEV), token_of.to(DEV), order.to(DEV)
+        xq, xs = quantize_mx(x.to(DEV))
+        hq = torch.zeros(m, hid, device=DEV, dtype=F8)
+        hs = torch.zeros(m, hid // 32, device=DEV, dtype=torch.uint8)
+        pre = torch.zeros(m, 2 * hid, device=DEV, dtype=torch.bfloat16)
+        launch_gemm1(xq, xs, tok_d, *packed.in_fwd, hq, hs, pre, off_d, hid, dim, torch.bfloat16)
+        dq, ds = quantize_mx(dout)
+        mpad = padded_rows(m, e)
+
+        def run(with_dpre, with_tok):
+            dpre = torch.zeros(m, 2 * hid, device=DEV, dtype=torch.bfloat16) if with_dpre else None
+            dpq = torch.zeros(m, 2 * hid, device=DEV, dtype=F8)
+            dps = torch.zeros(m, 2 * hid // 32, device=DEV, dtype=torch.uint8)
+            dgate = torch.zeros(tokens, device=DEV, dtype=torch.float32)
+            ptq = torch.zeros(2 * hid, mpad, device=DEV, dtype=F8) if with_tok else None
+            pts = torch.zeros(2 * hid, mpad // 32, device=DEV, dtype=torch.uint8) if with_tok else None
+            launch_gemm2_dgrad(dq, ds, tok_d, ord_d, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, off_d,
+                               ptq, pts)
+            return dpre, dpq, dps, dgate, ptq, pts
+
+        dpre0, dpq0, dps0, dgate0, _, _ = run(True, False)
+        dpre1, dpq1, dps1, dgate1, ptq1, pts1 = run(True, True)
+        _, dpq2, dps2, dgate2, ptq2, pts2 = run(False, True)
+        for a, b in ((dpre0, dpre1), (dpq0, dpq1), (dps0, dps1), (dpq0, dpq2), (dps0, dps2), (ptq1, ptq2), (pts1, pts2)):
+            assert torch.equal(a.view(torch.uint8) if a.dtype == F8 else a, b.view(torch.uint8) if b.dtype == F8 else b)
+        # dgate is an fp32 atomic sum: order-dependent in the last bits
+        assert torch.allclose(dgate0, dgate1, rtol=1e-4, atol=1e-6) and torch.allclose(dgate0, dgate2, rtol=1e-4, atol=1e-6)
+        rq, rs = quantize_mx_cols_grouped(dpre0, off_d, m)
+        valid = torch.zeros(mpad, dtype=torch.bool)
+        pos = 0
+        for c in counts:
+            tiles = -(-c // 128)
+            valid[pos : pos + tiles * 128] = True
+            pos += tiles * 128
+        assert torch.equal(ptq1.view(torch.uint8).cpu()[:, valid], rq.view(torch.uint8).cpu()[:, valid])
+        assert torch.equal(pts1.cpu()[:, valid.view(-1, 32)[:, 0]], rs.cpu()[:, valid.view(-1, 32)[:, 0]])
+        assert not ptq1.view(torch.uint8).cpu()[:, ~valid].any()  # nothing is written past the experts' tiles
+        with pytest.raises(Exception):
+            run(False, False)  # neither output asked for
+
+
 def test_expert_call_contract():
     from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, mxfp8_moe_experts
 
