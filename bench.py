@@ -279,6 +279,25 @@ def build_workload(name: str, dev):
 
         n = x_h.shape[0]
         return step, 2 * 2.0 * n**3 / 1e9, "outlier-stress 8192^3 GEMM, fwd + wgrad, quantizers included (BASELINE configs[4])", refresh
+    if name == "norm":
+        from kohakuwullm_amd.kernels.elementwise import rms_norm_mx
+
+        g = torch.Generator().manual_seed(SEED)
+        tokens, dim = 32768, 2048  # the hidden-state matrix of BASELINE configs[2]
+        x_h = torch.randn(tokens, dim, generator=g).bfloat16()
+        w_h = (1.0 + 0.1 * torch.randn(dim, generator=g)).bfloat16()
+        dy_h = (torch.randn(tokens, dim, generator=g) * 1e-2).bfloat16()
+        xs = [x_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
+        dys = [dy_h.to(dev) for _ in range(ncopies)]
+        w = w_h.to(dev).requires_grad_(True)
+
+        def step(i):
+            x = xs[i % ncopies]
+            out, q, s = rms_norm_mx(x, w, 1e-6)
+            out.backward(dys[i % ncopies])
+            x.grad = w.grad = None
+
+        return step, 0.0, "RMSNorm -> (bf16 out, MXFP8 pair) fwd + bwd on the 32768 x 2048 hidden states of BASELINE configs[2] (scope row 'next' 1)", lambda: None
     raise SystemExit(f"unknown workload {name!r}")
 
 
@@ -287,7 +306,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier"),
+    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm"),
                     help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
@@ -350,8 +369,21 @@ def main() -> None:
     quant = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n not in GEMM_ENTRIES]
     gemm_flops, gemm_ms = sum(w for _, w, _ in gemm), sum(t for _, _, t in gemm)
     quant_bytes, quant_ms = sum(w for _, w, _ in quant), sum(t for _, _, t in quant)
-    gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
     quant_gbs = quant_bytes / (quant_ms * 1e-3) / 1e9
+    if not gemm:
+        # a workload of streaming kernels only: the figure of merit is bytes per second against HBM
+        step_bytes = quant_bytes / args.steps
+        print(json.dumps({
+            "metric": "RMSNorm -> MXFP8 producer fwd+bwd GB/s", "value": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 arithmetic on bf16, fp64 sum of squares",
+            "data": "synthetic", "config": {"workload": desc, "bytes_per_step": int(step_bytes)},
+            "roofline": {"kernel": ", ".join(sorted({n for n, _, _ in quant})), "bound": "hbm", "achieved": round(quant_gbs, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "launches": len(quant), "avg_launch_us": round(quant_ms / len(quant) * 1e3, 2)},
+        }))
+        return
+    gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
 
     out = {
         "metric": "MXFP8 linear fwd+bwd TFLOP/s (quantizers included)",

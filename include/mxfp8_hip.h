@@ -122,6 +122,34 @@ int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, in
                                 uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
 
 /*
+ * RMSNorm as a producer of MXFP8 operands: rstd[m] = 1 / sqrt(mean_k(x[m,k]^2) + eps),
+ * y = x * rstd * weight (fp32; weight NULL: 1).  Any of three results, from one pass over x:
+ * out (M,K) in x_dtype (NULL: not written), rstd (M) fp32 for the backward (NULL: not
+ * written), and (q,s) = y quantized along K from the fp32 values (both NULL: not written;
+ * K % 32 == 0 when given).  At least one of out and q.  weight is x_dtype or fp32.
+ * The sum of squares is accumulated in fp64, the rest is fp32 in the reference's order.
+ * Replaces _rmsnorm_fwd with QUANT (src/kohakuwullm/kernels/elementwise/rmsnorm.py:20-84;
+ * host side rms_norm_mx :239-246, rms_norm :232-236) and _rmsnorm_mx_kernel / rmsnorm_mx
+ * (src/kohakuwullm/kernels/mxfp8/fused_act.py:104-175).  The SWIZZLE branch of the reference
+ * is mx_swizzle_scales applied to s.
+ */
+int mx_rmsnorm_quantize(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                        const void *weight, int w_dtype, float eps, void *out, int64_t ldo, float *rstd,
+                        uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream);
+
+/*
+ * RMSNorm backward: dx = (dy - xhat * mean_k(dy * xhat)) * rstd with dy = dout * weight and
+ * xhat = x * rstd, in dtype (bf16 or fp16); dw_part (parts,K) fp32 (NULL: no weight
+ * gradient) receives one partial sum of dout * xhat per workgroup, every row of it written;
+ * the caller adds the rows.  1 <= parts <= 65535; K <= 4096.
+ * Replaces _rmsnorm_bwd (src/kohakuwullm/kernels/elementwise/rmsnorm.py:87-128, launched
+ * from _RMSNorm.backward :196-229 with 512 partial rows).
+ */
+int mx_rmsnorm_backward(const void *x, int dtype, int64_t M, int64_t K, int64_t ldx, const void *weight,
+                        int w_dtype, const void *dout, int64_t lddo, const float *rstd, void *dx, int64_t lddx,
+                        float *dw_part, int64_t parts, void *stream);
+
+/*
  * Scale layout interop.  The reference's cuBLAS route keeps UE8M0 scales in the flat
  * SWIZZLE_32_4_4 layout: 128-row x 4-column tiles of 512 bytes, row-tile major, scale
  * (r, c) of a tile at (r % 32) * 16 + (r / 32) * 4 + c, zero padded to whole tiles

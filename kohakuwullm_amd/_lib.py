@@ -50,6 +50,10 @@ SIGNATURES = {
         _ci, [_p, _ci, _i64, _i64, _ci, _p, _p, _ci, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_grouped_wgrad_nt": (
         _ci, [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p]),
+    "mx_rmsnorm_quantize": (
+        _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, ctypes.c_float, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
+    "mx_rmsnorm_backward": (
+        _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
     "mx_swizzle_scales": (_ci, [_p, _i64, _i64, _i64, _p, _p]),
     "mx_unswizzle_scales": (_ci, [_p, _i64, _i64, _p, _i64, _p]),
     "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),

@@ -293,17 +293,10 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
         for (int j = 0; j < S::NT; j++) asm volatile("" : "+v"(acc[i][j]));
 }
 
-// s_waitcnt with lgkmcnt(0), no expcnt wait, and at most `n` vector-memory operations left in
-// flight (n <= 63).  Vector-memory operations retire in issue order, so this waits for
-// everything except the youngest n.
-__device__ __forceinline__ void wait_vm_allow(int n) {
-    // simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    switch (n) {
-    case 0: __builtin_amdgcn_s_waitcnt(0x0070); break;
-    case 1: __builtin_amdgcn_s_waitcnt(0x0071); break;
-    default: break;
-    }
-}
+// s_waitcnt with lgkmcnt(0), no expcnt wait, and at most N vector-memory operations left in
+// flight.  Vector-memory operations retire in issue order, so this waits for everything except
+// the youngest N.
+// simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
 template <int N>
 __device__ __forceinline__ void wait_vm_allow_c() {
     static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
@@ -362,7 +355,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
         if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
     }
-    wait_vm_allow(0);
+    wait_vm_allow_c<0>();
     __syncthreads();
 
     v4f acc[S::MT][S::NT];
@@ -416,7 +409,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             compute_stage<S, SIDX>(ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64, b_rd,     \
                                    b_rd ^ 64, sa, sb, acc, ctx, L, kt_issue, ldsA, ldsB, buf ^ 1);            \
             if (!last) {                                                                                      \
-                wait_vm_allow(0);                                                                             \
+                wait_vm_allow_c<0>();                                                                         \
                 __syncthreads();                                                                              \
             }                                                                                                 \
             gstage++;                                                                                         \
@@ -442,7 +435,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         }
         if (!has_next) break;
         if (stores == P::NST) wait_vm_allow_c<P::NST>();
-        else wait_vm_allow(0);
+        else wait_vm_allow_c<0>();
         __syncthreads();
         cur = nxt;
         has_next = prob.next(nxt);

@@ -16,6 +16,8 @@ Reference lines followed (paths relative to the reference tree):
   ``src/kohakuwullm/kernels/mxfp8/moe.py:408-433``
 * error metrics ........... ``src/kohakuwullm/bench/core/timing.py:201-228``
 * expert sort (CPU) ....... ``src/kohakuwullm/kernels/moe/moe_dispatch.py:264-282``
+* RMSNorm -> MXFP8 ........ ``src/kohakuwullm/kernels/elementwise/rmsnorm.py:20-128``,
+  ``src/kohakuwullm/kernels/mxfp8/fused_act.py:104-143``
 
 All tensors are CPU tensors.  Codes travel as ``torch.uint8`` (bit patterns of
 ``float8_e4m3fn``) unless stated otherwise.
@@ -251,3 +253,42 @@ def expert_sort(flat_expert: torch.Tensor, num_experts: int, top_k: int):
 
 def silu(x: torch.Tensor) -> torch.Tensor:
     return x * torch.sigmoid(x)
+
+
+# --------------------------------------------------------------------------- RMSNorm producer
+
+
+def rms_norm_mx(x: torch.Tensor, weight: torch.Tensor | None, eps: float = 1e-6):
+    """``(out, rstd, q, s)`` of ``_rmsnorm_fwd`` with QUANT (rmsnorm.py:52-84).
+
+    ``rstd = 1 / sqrt(sum(x^2) / K + eps)`` with the sum taken in fp64 (exact for 16-bit inputs, so
+    every summation order agrees on the fp32 it rounds to) and the remaining steps in fp32 in the
+    reference's order; ``y = x * rstd * w`` in fp32; ``out`` is ``y`` rounded to ``x.dtype``; the
+    codes are quantized from the fp32 ``y`` (K % 32 == 0, else ``q = s = None``).
+    """
+    import numpy as np
+
+    m, k = x.shape
+    ss = x.double().square().sum(dim=1).numpy()
+    # each fp32 step as "fp64 operation, rounded once to fp32": for fp32 operands that is the correctly
+    # rounded fp32 result (53 >= 2 * 24 + 2 bits) and it does not depend on which vector code path a
+    # CPU build of torch picks for float sqrt and divide (they were seen to differ between hosts)
+    mean = (ss.astype(np.float32).astype(np.float64) / np.float64(np.float32(k))).astype(np.float32) + np.float32(eps)
+    root = np.sqrt(mean.astype(np.float64)).astype(np.float32)
+    rstd = torch.from_numpy((1.0 / root.astype(np.float64)).astype(np.float32))
+    y = x.float() * rstd[:, None]
+    if weight is not None:
+        y = y * weight.float()[None, :]
+    q = s = None
+    if k % BLOCK_SCALE == 0:
+        q, s = quantize_rows(y.contiguous())
+    return y.to(x.dtype), rstd, q, s
+
+
+def rms_norm_grads(x: torch.Tensor, weight: torch.Tensor | None, dout: torch.Tensor, eps: float = 1e-6):
+    """``(dx, dw)`` in fp64 by automatic differentiation of torch's own ``rms_norm`` (rmsnorm.py:87-128 computes the same)."""
+    xd = x.double().requires_grad_(True)
+    wd = None if weight is None else weight.double().requires_grad_(True)
+    out = torch.nn.functional.rms_norm(xd, (x.shape[1],), wd, eps)
+    out.backward(dout.double())
+    return xd.grad, None if wd is None else wd.grad
