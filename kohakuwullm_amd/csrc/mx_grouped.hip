@@ -730,42 +730,24 @@ struct WgradProblem {
         int slot;  // fp32 scratch slot of this K slice, or -1 for a whole tile
     };
     const WgradArgs p;
-    // Units are dealt round-robin over the workgroups: first the (tile, K slice) units of the
-    // non-empty experts, compactly numbered so they spread evenly wherever those experts sit
-    // among the E, then the tiles of the empty experts, which are only zero-filled.
-    int next_unit, next_dead, kb_end;
+    // Units are dealt round-robin over the workgroups: the (tile, K slice) units of the non-empty
+    // experts, compactly numbered so they spread evenly wherever those experts sit among the E.
+    // (The dW of an expert without rows is zero-filled by wgrad_zero_kernel, launched first.)
+    int next_unit, kb_end;
     int live, slices;
-    // incremental scans: expert scan_e is the scan_live-th non-empty one and its first K stage
-    // is scan_tiles; expert dead_e is the dead_seen-th empty one
-    int scan_e, scan_tiles, scan_live, dead_e, dead_seen;
+    // incremental scan: expert scan_e is the scan_live-th non-empty one and its first K stage
+    // is scan_tiles
+    int scan_e, scan_tiles, scan_live;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
-    __device__ WgradProblem(const WgradArgs &a)
-        : p(a), next_unit(blockIdx.x), next_dead(blockIdx.x), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0),
-          dead_e(0), dead_seen(0) {
-        slices = wgrad_slices(p, (int)gridDim.x, live);
-    }
-
-    __device__ __forceinline__ void zero_tile(int expert, int m0, int n0) const {
-        // an expert without rows: its dW tile is zeros
-        const int esz = CDT == MX_FP32 ? 4 : 2;
-        char *base = (char *)p.dw + (int64_t)expert * p.stride_dwe * esz;
-        if (p.c_vec && m0 + S::BM <= p.N && n0 + S::BN <= p.Kout) {
-            constexpr int PER_ROW = S::BN * esz / 16;
-            for (int idx = threadIdx.x; idx < S::BM * PER_ROW; idx += S::NTHR) {
-                const int m = m0 + idx / PER_ROW, c = idx % PER_ROW;
-                *(v4i *)(base + ((int64_t)m * p.lddw + n0) * esz + c * 16) = v4i{0, 0, 0, 0};
-            }
-            return;
-        }
-        for (int idx = threadIdx.x; idx < S::BM * S::BN; idx += S::NTHR) {
-            const int m = m0 + idx / S::BN, n = n0 + idx % S::BN;
-            if (m < p.N && n < p.Kout) {
-                char *dst = base + ((int64_t)m * p.lddw + n) * esz;
-                if (esz == 4) *(float *)dst = 0.0f;
-                else *(uint16_t *)dst = 0;
-            }
-        }
+    // Workgroups are dealt to the 8 XCDs round-robin, so workgroup b starts at unit
+    // (b % 8) * (G / 8) + b / 8: the workgroups of one XCD take consecutive units, i.e. the tiles
+    // of one (expert, K slice), which read the same operand panels, share that XCD's L2 (measured:
+    // the kernel's fabric reads equal the operand bytes).
+    __device__ WgradProblem(const WgradArgs &a) : p(a), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0) {
+        const int g = (int)gridDim.x, b = (int)blockIdx.x;
+        next_unit = (g & 7) == 0 ? (b & 7) * (g >> 3) + (b >> 3) : b;
+        slices = wgrad_slices(p, g, live);
     }
 
     __device__ __forceinline__ void zero_slot(int slot) const {
@@ -804,18 +786,6 @@ struct WgradProblem {
                 continue;
             }
             return true;
-        }
-        const int dead_tiles = (p.E - live) * per_e;
-        while (next_dead < dead_tiles) {
-            const int d = next_dead / per_e, rem = next_dead - d * per_e;
-            next_dead += gridDim.x;
-            while (true) {
-                const bool empty = p.offsets[dead_e + 1] <= p.offsets[dead_e];
-                if (empty && dead_seen == d) break;
-                dead_seen += empty ? 1 : 0;
-                dead_e++;
-            }
-            zero_tile(dead_e, (rem / p.tiles_n) * S::BM, (rem % p.tiles_n) * S::BN);
         }
         return false;
     }
@@ -875,6 +845,32 @@ struct WgradProblem {
         return interior ? NST : -1;
     }
 };
+
+// dW of the experts without rows: zeros.  A plain streaming fill, launched ahead of the GEMM (as
+// part of it, the fills of 58 empty experts cost three times what they cost here).  One block
+// per (expert, 64 rows).
+template <int CDT>
+__global__ __launch_bounds__(256) void wgrad_zero_kernel(WgradArgs p, int chunks) {
+    const int e = blockIdx.x / chunks, m0 = (blockIdx.x % chunks) * 64;
+    if (p.offsets[e + 1] > p.offsets[e]) return;
+    const int esz = CDT == MX_FP32 ? 4 : 2;
+    char *base = (char *)p.dw + ((int64_t)e * p.stride_dwe + (int64_t)m0 * p.lddw) * esz;
+    const int rows = p.N - m0 < 64 ? p.N - m0 : 64;
+    if (p.c_vec && (p.Kout * esz) % 16 == 0) {
+        const int per_row = p.Kout * esz / 16;
+        for (int idx = threadIdx.x; idx < rows * per_row; idx += 256) {
+            const int m = idx / per_row, c = idx - m * per_row;
+            *(v4i *)(base + (int64_t)m * p.lddw * esz + c * 16) = v4i{0, 0, 0, 0};
+        }
+        return;
+    }
+    for (int idx = threadIdx.x; idx < rows * p.Kout; idx += 256) {
+        const int m = idx / p.Kout, n = idx - m * p.Kout;
+        char *dst = base + ((int64_t)m * p.lddw + n) * esz;
+        if (esz == 4) *(float *)dst = 0.0f;
+        else *(uint16_t *)dst = 0;
+    }
+}
 
 template <typename S, int CDT>
 __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) {
@@ -1126,6 +1122,9 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
     dim3 grid((unsigned)(work * (a.slots ? 8 : 1) < cus ? work * (a.slots ? 8 : 1) : cus)), block(S::NTHR);
     auto kern = grouped_wgrad_kernel<S, CDT>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
+    const int chunks = (a.N + 63) / 64;
+    if ((int64_t)a.E * chunks >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    wgrad_zero_kernel<CDT><<<dim3((unsigned)(a.E * chunks)), dim3(256), 0, st>>>(a, chunks);
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
     if (a.slots) wgrad_reduce_kernel<S, CDT><<<dim3((unsigned)(work * S::MT)), block, 0, st>>>(a, (int)grid.x);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;

@@ -104,6 +104,18 @@ def padded_rows(rows: int, num_experts: int) -> int:
     return (-(-rows // WGRAD_ROW_TILE) + num_experts) * WGRAD_ROW_TILE
 
 
+# Extra bytes in the row pitch of the token-axis code buffers, see `token_axis_buffers`.
+TOKEN_PITCH_PAD = 0
+
+
+def token_axis_buffers(cols: int, mpad: int, device):
+    """``(cols, mpad)`` codes and ``(cols, mpad // 32)`` scales for a token-axis quantization, as views of wider rows."""
+    pitch = mpad + TOKEN_PITCH_PAD
+    qt = torch.empty(cols, pitch, device=device, dtype=_FP8)[:, :mpad]
+    st = torch.empty(cols, mpad // BLOCK_SCALE, device=device, dtype=torch.uint8)
+    return qt, st
+
+
 def quantize_mx_cols_grouped(
     x: torch.Tensor,
     offsets: torch.Tensor,
@@ -129,15 +141,14 @@ def quantize_mx_cols_grouped(
     _lib.require_gpu(x, "x")
     cols = x.shape[1] // 2 if swiglu else x.shape[1]
     mpad = padded_rows(rows, num_experts)
-    qt = torch.empty(cols, mpad, device=x.device, dtype=_FP8)
-    st = torch.empty(cols, mpad // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+    qt, st = token_axis_buffers(cols, mpad, x.device)
     scale_dt = 0 if row_scale is None else _lib.MX_DTYPE[row_scale.dtype]
     _lib.invoke(
         "mx_quantize_cols_grouped", rows * cols * ((4 if swiglu else 2) + 1 + 1 / BLOCK_SCALE), x,
         x.data_ptr(), _lib.MX_DTYPE[x.dtype], x.stride(0), cols, 1 if swiglu else 0,
         0 if index is None else index.data_ptr(), 0 if row_scale is None else row_scale.data_ptr(), scale_dt,
         0 if scale_index is None else scale_index.data_ptr(), offsets.data_ptr(), num_experts, rows,
-        qt.data_ptr(), mpad, st.data_ptr(), mpad // BLOCK_SCALE,
+        qt.data_ptr(), qt.stride(0), st.data_ptr(), st.stride(0),
     )
     return qt, st
 

@@ -20,6 +20,7 @@ from kohakuwullm_amd.kernels.mxfp8.grouped import (
     grouped_mxfp8_gemm,
     grouped_mxfp8_wgrad,
     padded_rows,
+    token_axis_buffers,
     quantize_mx_cols_grouped,
 )
 from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE, quantize_mx, quantize_mx_cols
@@ -177,8 +178,7 @@ class _MXFP8Experts(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             # h along the tokens, for dW_out: written by GEMM1's epilogue instead of a pass over `pre`
             mpad = padded_rows(m, packed.in_fwd[0].shape[0])
-            htq = torch.empty(hidden, mpad, device=x.device, dtype=_FP8)
-            hts = torch.empty(hidden, mpad // BLOCK_SCALE, device=x.device, dtype=torch.uint8)
+            htq, hts = token_axis_buffers(hidden, mpad, x.device)
         launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hidden, dim, x.dtype, htq, hts)
         # pairs per token when `order` is the pair index token * top_k + slot; 0 = unknown layout
         top_k = gate.numel() // rows if rows and gate.numel() % rows == 0 else 0
@@ -205,8 +205,7 @@ class _MXFP8Experts(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             # dpre along the tokens, for dW_in: written by the epilogue; dpre itself never reaches memory
             mpad = padded_rows(m, packed.in_fwd[0].shape[0])
-            ptq = torch.empty(2 * hidden, mpad, device=dev, dtype=_FP8)
-            pts = torch.empty(2 * hidden, mpad // BLOCK_SCALE, device=dev, dtype=torch.uint8)
+            ptq, pts = token_axis_buffers(2 * hidden, mpad, dev)
         dpre = None if ptq is not None else torch.empty(m, 2 * hidden, device=dev, dtype=dout.dtype)
         launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets,
                            ptq, pts)
