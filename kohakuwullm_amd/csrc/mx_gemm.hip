@@ -34,6 +34,9 @@ struct DenseArgs {
     float *sk_ws;
 };
 
+// Whether tile_of staggers the column walk (see there): up to 64 K stages per tile.
+__host__ __device__ inline bool stagger_columns(int64_t K) { return K <= 64 * 128; }
+
 template <typename S, int CDT>
 struct DenseProblem {
     struct Tile {
@@ -63,7 +66,7 @@ struct DenseProblem {
             const int k0 = sk_pos - local * KT4;
             const int stop = k0 + (sk_end - sk_pos);
             int tm, tn;
-            tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn);
+            tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
             t.m0 = tm * S::BM;
             t.n0 = tn * S::BN;
             t.kt0 = k0;
@@ -79,7 +82,7 @@ struct DenseProblem {
         const int slice = next_id / per_slice;
         const int index = next_id - slice * per_slice;
         int tm, tn;
-        tile_of(index, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
         t.slot = p.slice_ws ? index * p.split_k + slice : -1;
         t.m0 = tm * S::BM;
         t.n0 = tn * S::BN;
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
         for (int j = 0; j < S::NT; j++) sum[j] += src[(i * S::NT + j) * S::NTHR + tid];
     }
     int tm, tn;
-    tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn);
+    tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WGN, wn = wave % S::WGN;
     const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
@@ -267,7 +270,7 @@ __global__ __launch_bounds__(S::NTHR) void slice_reduce_kernel(DenseArgs p) {
         for (int j = 0; j < S::NT; j++) sum[j] += src[(i * S::NT + j) * S::NTHR + tid];
     }
     int tm, tn;
-    tile_of(index, p.tiles_m, p.tiles_n, tm, tn);
+    tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WGN, wn = wave % S::WGN;
     const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
