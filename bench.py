@@ -238,10 +238,12 @@ def build_workload(name: str, dev):
             proj.refresh_quantized_weight()
 
         def step(i):
-            x = xs[i % ncopies]
+            # the attention core is not run: o_proj sees another activation of the same shape (its own
+            # tensor, as in a block, so autograd has no second dX to add into the first)
+            x, a = xs[i % ncopies], xs[(i + 2) % ncopies]
             qkv(x).backward(d_qkv)
-            proj(x).backward(d_o)  # the attention core is not run: o_proj sees an activation of the same shape
-            x.grad = qkv.weight.grad = proj.weight.grad = None
+            proj(a).backward(d_o)
+            x.grad = a.grad = qkv.weight.grad = proj.weight.grad = None
 
         t, d = hid_h.shape
         gflop = 3 * (2.0 * t * w_qkv_h.shape[0] * d + 2.0 * t * d * d) / 1e9

@@ -494,7 +494,23 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         mode = scale_mode(a) > mode ? scale_mode(a) : mode;
         tiles[j] = a.dp_tiles;
         KT[j] = ((a.K + 127) >> 7);
-        alone += (tiles[j] + cus - 1) / cus * (KT[j] + 4);
+        // a launch of its own: whole rounds of tiles, then the last round with the same even K
+        // split launch_tiled would choose
+        const int64_t rest = tiles[j] % cus, KT4 = (KT[j] + 3) & ~3;
+        alone += tiles[j] / cus * (KT[j] + 4);
+        if (rest) {
+            int64_t q = (rest * KT4 + cus - 1) / cus;
+            q = ((q < KT4 / 8 ? KT4 / 8 : q) + 3) & ~(int64_t)3;
+            const double pieces = (double)rest * KT4 / q + rest, cost = 4.0 + 0.15 * pieces;
+            alone += KT4 >= 8 && (double)(KT4 - q) > 1.25 * cost ? q + (int64_t)cost : KT[j] + 4;
+        }
+        // A product with several full rounds of tiles runs well on its own (each XCD's 32 CUs
+        // share A/B panels in L2, the ragged last round is K-split); confined to a part of the
+        // GPU beside another product it shares less and both become bound by HBM.  Measured
+        // with operands that are not cache-resident: 32768 x 2048 x 3072 beside its weight
+        // gradient 479 us in one launch, 404 us one after the other; the three backward
+        // products of the feed-forward block (1.5, 0.75 and 0.4 rounds) 482 against 536.
+        if (tiles[j] >= 2 * (int64_t)cus) fuse = false;
     }
     int share[MX_BATCH_MAX], slices[MX_BATCH_MAX], best_share[MX_BATCH_MAX], best_slices[MX_BATCH_MAX];
     int64_t best = -1;
