@@ -299,7 +299,7 @@ def build_workload(name: str, dev):
             out.backward(dys[i % ncopies])
             x.grad = w.grad = None
 
-        return step, 0.0, "RMSNorm -> (bf16 out, MXFP8 pair) fwd + bwd on the 32768 x 2048 hidden states of BASELINE configs[2] (scope row 'next' 1)", lambda: None
+        return step, 0.0, "RMSNorm -> (bf16 out, MXFP8 pair) fwd + bwd on the 32768 x 2048 hidden states of BASELINE configs[2]", lambda: None
     raise SystemExit(f"unknown workload {name!r}")
 
 
