@@ -211,6 +211,37 @@ def test_gemm_batch(oracle, shapes, dtype):
     assert _mx().mxfp8_matmul_pq_batch([], dtype) == []
 
 
+# Many tiles: the walk over the tile grid (XCD ranges, row groups of 4, staggered columns for
+# short K, plain order for long K) must visit every tile exactly once whatever the grid's shape.
+WALK_SHAPES = [
+    (1300, 2300, 256),  # 6 x 9 tiles: a ragged last row group, more columns than XCDs
+    (3000, 600, 1024),  # 12 x 3: fewer columns than XCDs
+    (2560, 5000, 512),  # 10 x 20
+    (4100, 260, 128),  # 17 x 2
+    (1030, 4000, 8192),  # 5 x 16, K at the stagger limit
+    (1030, 4000, 8320),  # just past it: columns walked in order
+    (257, 257, 384),  # 2 x 2 with one-element edge tiles
+]
+
+
+@pytest.mark.parametrize("m,n,k", WALK_SHAPES)
+def test_gemm_tile_walk_covers_every_tile(oracle, m, n, k):
+    aq, as_, bq, bs = _operands(oracle, m, n, k, seed=SEED + m + n)
+    ref = oracle.gemm_nt(aq, as_, bq, bs)
+    # the output buffer starts as NaN: a tile the walk skipped stays NaN (one visited twice is harmless
+    # to the value, so coverage is what this adds); values are checked against the oracle as everywhere
+    from kohakuwullm_amd.kernels.mxfp8.quantize import _gemm_nt_into
+
+    f8 = torch.float8_e4m3fn
+    out = torch.full((m, n), float("nan"), device=DEV, dtype=torch.bfloat16)
+    _gemm_nt_into(aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV), out)
+    got = out.cpu()
+    assert torch.isfinite(got).all()
+    assert oracle.rel_error(got, ref) < TOL_BF16
+    tile_err = (got.double() - ref).abs().view(-1)
+    assert tile_err.max().item() <= 0.02 * ref.abs().max().item() + 1e-6
+
+
 def test_gemm_unaligned_operands_take_the_generic_kernel(oracle):
     """Row pitches that are not multiples of 16 bytes cannot feed the copy engine: the slow kernel serves them."""
     m, n, k = 96, 80, 256
