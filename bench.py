@@ -188,7 +188,7 @@ def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
 # Bytes the GEMM launches of one step move between the L2s and the fabric, per launch, from the
 # FETCH_SIZE and WRITE_SIZE counter runs summarised under profiles/ (each scaled by what the
 # counter reads for a device copy of known size): 3090 MiB over 4 launches.
-GEMM_TRAFFIC_PER_LAUNCH = {"ffn": 776 * 2**20}
+GEMM_TRAFFIC_PER_LAUNCH = {"ffn": 521 * 2**20}
 
 GEMM_ENTRIES = ("mx_gemm_nt", "mx_gemm_nt_batch", "mx_grouped_gemm_nt", "mx_experts_gemm1", "mx_experts_scatter_gemm",
                 "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt")

@@ -32,6 +32,7 @@ struct DenseArgs {
     // measured slower: one CU pulls the other pieces at ~40 GB/s, a kernel of its own at TB/s.)
     int dp_tiles, sk_tiles, sk_q;
     float *sk_ws;
+    int xcds;  // XCDs this problem's workgroups are spread over (8; fewer inside a batched launch)
 };
 
 // Whether tile_of staggers the column walk (see there): up to 64 K stages per tile.
@@ -66,7 +67,7 @@ struct DenseProblem {
             const int k0 = sk_pos - local * KT4;
             const int stop = k0 + (sk_end - sk_pos);
             int tm, tn;
-            tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
+            tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K), p.xcds);
             t.m0 = tm * S::BM;
             t.n0 = tn * S::BN;
             t.kt0 = k0;
@@ -82,7 +83,7 @@ struct DenseProblem {
         const int slice = next_id / per_slice;
         const int index = next_id - slice * per_slice;
         int tm, tn;
-        tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
+        tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K), p.xcds);
         t.slot = p.slice_ws ? index * p.split_k + slice : -1;
         t.m0 = tm * S::BM;
         t.n0 = tn * S::BN;
@@ -199,22 +200,29 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
     persistent_gemm<S, K512>(prob, smem);
 }
 
-// Several independent products in one launch.  The workgroups are partitioned among the
-// problems (cu_lo[j] .. cu_lo[j+1]) in proportion to their work, so a product with too few
+// Several independent products in one launch.  The XCDs are partitioned among the problems
+// (x_lo[j] .. x_lo[j+1]) in proportion to their work, so a product with too few
 // tiles to fill the GPU runs beside the others instead of leaving most of it idle.
 #define MX_BATCH_MAX 4
+// Problem j owns XCDs [x_lo[j], x_lo[j + 1]) whole: all 32 CUs of an XCD then work on one product
+// and share its panels in that XCD's L2.  (Dealing every problem a few CUs of every XCD instead
+// was measured: the three backward products of the feed-forward block pulled 1957 MiB through
+// the fabric in 490 us, which is the part's bandwidth.)
 struct DenseBatchArgs {
     DenseArgs prob[MX_BATCH_MAX];
-    int cu_lo[MX_BATCH_MAX + 1];
+    int x_lo[MX_BATCH_MAX + 1];
     int count;
 };
 
 template <typename S, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    // workgroups go to the XCDs round-robin: this one runs on XCD blockIdx.x % 8
+    const int x = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
     int j = 0;
-    while (j + 1 < b.count && (int)blockIdx.x >= b.cu_lo[j + 1]) j++;
-    DenseProblem<S, CDT> prob(b.prob[j], (int)blockIdx.x - b.cu_lo[j], b.cu_lo[j + 1] - b.cu_lo[j]);
+    while (j + 1 < b.count && x >= b.x_lo[j + 1]) j++;
+    const int nx = b.x_lo[j + 1] - b.x_lo[j];
+    DenseProblem<S, CDT> prob(b.prob[j], (x - b.x_lo[j]) + nx * slot, nx * ((int)gridDim.x >> 3));
     persistent_gemm<S, K512>(prob, smem);
 }
 
@@ -240,7 +248,7 @@ __global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
         for (int j = 0; j < S::NT; j++) sum[j] += src[(i * S::NT + j) * S::NTHR + tid];
     }
     int tm, tn;
-    tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
+    tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K), p.xcds);
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WGN, wn = wave % S::WGN;
     const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
@@ -270,7 +278,7 @@ __global__ __launch_bounds__(S::NTHR) void slice_reduce_kernel(DenseArgs p) {
         for (int j = 0; j < S::NT; j++) sum[j] += src[(i * S::NT + j) * S::NTHR + tid];
     }
     int tm, tn;
-    tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K));
+    tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K), p.xcds);
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WGN, wn = wave % S::WGN;
     const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
@@ -463,20 +471,19 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
     return launch_tiled<DenseShape, CDT>(a, st);
 }
 
-// Several products behind one launch, the workgroups shared out among them in groups of 8 (one
-// per XCD, so each problem's tile order keeps its XCD locality).  A group goes, one at a time,
-// to the problem that would otherwise finish last; cost of a problem on n workgroups =
-// rounds of tiles x (K stages + 4 for the tile's prologue and epilogue).  A problem with few,
-// long tiles (a weight gradient) may in addition be cut into 2 or 4 K slices that run as
-// independent tiles and leave fp32 partial sums for slice_reduce_kernel; every combination of
-// slice counts is priced (a partial tile costs about 0.1 stage of everyone's time) and the
-// cheapest plan wins, against running the products one after the other as well.
+// Several products behind one launch, the eight XCDs shared out among them whole.  Every problem
+// gets one XCD, the rest go, one at a time, to the problem that would otherwise finish last; cost
+// of a problem on n workgroups = rounds of tiles x (K stages + 4 for the tile's prologue and
+// epilogue).  A problem with few, long tiles (a weight gradient) may in addition be cut into 2 or
+// 4 K slices that run as independent tiles and leave fp32 partial sums for slice_reduce_kernel;
+// every combination of slice counts is priced (a partial tile costs about 0.1 stage of
+// everyone's time) and the cheapest plan wins, against running the products one after the other
+// as well.
 template <int CDT>
 static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     typedef DenseShape S;
     const int cus = num_cus();
-    const int groups = cus / 8;
-    bool fuse = count > 1 && count <= MX_BATCH_MAX && groups >= count && split_mode();
+    bool fuse = count > 1 && count <= MX_BATCH_MAX && split_mode();
     DenseBatchArgs b;
     int64_t tiles[MX_BATCH_MAX], alone = 0;
     int KT[MX_BATCH_MAX];
@@ -512,13 +519,19 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         // products of the feed-forward block (1.5, 0.75 and 0.4 rounds) 482 against 536.
         if (tiles[j] >= 2 * (int64_t)cus) fuse = false;
     }
+    // Plan: a number of whole XCDs for every problem (they add up to 8) and a number of K slices,
+    // chosen together by pricing every combination.
     int share[MX_BATCH_MAX], slices[MX_BATCH_MAX], best_share[MX_BATCH_MAX], best_slices[MX_BATCH_MAX];
     int64_t best = -1;
+    fuse = fuse && cus % 8 == 0 && count <= 8;
     if (fuse) {
+        const int per_xcd = cus / 8;
         const int slots = 2 * cus;  // fp32 tile slots of the scratch
         auto per_slice = [&](int j) { return (((KT[j] + slices[j] - 1) / slices[j]) + 3) & ~3; };
         auto units = [&](int j) { return tiles[j] * slices[j]; };
-        auto finish = [&](int j) { return (units(j) + 8 * share[j] - 1) / (8 * share[j]) * (per_slice(j) + 4); };
+        auto finish = [&](int j) {
+            return (units(j) + per_xcd * share[j] - 1) / (per_xcd * share[j]) * (per_slice(j) + 4);
+        };
         int combos = 1;
         for (int j = 0; j < count; j++) combos *= 3;
         for (int code = 0; code < combos; code++) {
@@ -532,11 +545,11 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
                 share[j] = 1;
             }
             if (!ok || partial > slots) continue;
-            for (int left = groups - count; left > 0; left--) {
-                int worst = -1;
-                for (int j = 0; j < count; j++)
-                    if (8 * share[j] < units(j) && (worst < 0 || finish(j) > finish(worst))) worst = j;
-                if (worst < 0) break;
+            // the XCDs beyond one each go, one at a time, to the problem that would finish last
+            for (int left = 8 - count; left > 0; left--) {
+                int worst = 0;
+                for (int j = 1; j < count; j++)
+                    if (finish(j) > finish(worst)) worst = j;
                 share[worst]++;
             }
             int64_t together = partial ? 4 + partial / 10 : 0;
@@ -566,18 +579,17 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         }
         return MX_OK;
     }
-    b.cu_lo[0] = 0;
+    b.x_lo[0] = 0;
     int64_t slot_base = 0;
     for (int j = 0; j < count; j++) {
         DenseArgs &a = probs[j];
         a.split_k = best_slices[j];
+        a.xcds = best_share[j];
         if (a.split_k > 1) {
             a.slice_ws = scratch + slot_base * (S::BM * S::BN);
             slot_base += tiles[j] * a.split_k;
         }
-        const int64_t u = tiles[j] * a.split_k;
-        const int64_t wgs = 8 * best_share[j] < u ? 8 * best_share[j] : u;
-        b.cu_lo[j + 1] = b.cu_lo[j] + (int)wgs;
+        b.x_lo[j + 1] = b.x_lo[j] + best_share[j];
         b.prob[j] = a;
     }
     b.count = count;
@@ -585,7 +597,7 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
                 : mode == SCALES_DWORD ? gemm_nt_batch_kernel<S, CDT, SCALES_DWORD>
                                        : gemm_nt_batch_kernel<S, CDT, SCALES_BYTES>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
-    kern<<<dim3((unsigned)b.cu_lo[count]), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
+    kern<<<dim3((unsigned)cus), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
     for (int j = 0; j < count; j++)
         if (probs[j].split_k > 1)
             slice_reduce_kernel<S, CDT><<<dim3((unsigned)(tiles[j] * S::MT)), dim3(S::NTHR), 0, st>>>(probs[j]);
@@ -605,6 +617,7 @@ static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const u
     a.tiles_m = a.tiles_n = a.c_vec = 0;
     a.dp_tiles = a.sk_tiles = a.sk_q = 0;
     a.sk_ws = nullptr;
+    a.xcds = 8;
     return MX_OK;
 }
 

@@ -477,14 +477,15 @@ __device__ __forceinline__ void store8(void *c, int64_t off, const v4f &lo, cons
     }
 }
 
-// Maps a flat tile id to (tile_m, tile_n) so that (a) ids congruent mod 8 -- which run on the
-// same XCD, since workgroups are dealt to the 8 XCDs round-robin and the persistent stride is
-// a multiple of 8 -- are neighbours in tile space and share A/B panels in that XCD's L2, and
+// Maps a flat tile id to (tile_m, tile_n) so that (a) ids congruent mod `xcds` -- which run on
+// the same XCD: workgroups are dealt to the 8 XCDs round-robin, the persistent stride is a
+// multiple of 8, and a problem that owns only some of the XCDs (a batched launch) numbers its
+// workgroups XCD-fastest -- are neighbours in tile space and share A/B panels in that XCD's L2, and
 // (b) tiles are walked in column groups of GROUP_M row tiles.
-__device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &tm, int &tn, bool stagger) {
+__device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &tm, int &tn, bool stagger, int xcds) {
     const int total = tiles_m * tiles_n;
-    const int per_xcd = total >> 3;
-    if (id < (per_xcd << 3)) id = (id & 7) * per_xcd + (id >> 3);
+    const int per_xcd = total / xcds;
+    if (id < per_xcd * xcds) id = xcds == 8 ? (id & 7) * per_xcd + (id >> 3) : (id % xcds) * per_xcd + id / xcds;
     constexpr int GROUP_M = 4;  // measured in the training step: 4 beats 2, 6, 8 and 16 by 1-5 %
     const int width = GROUP_M * tiles_n;
     const int group = id / width;
@@ -493,7 +494,7 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &t
     const int in = id - group * width;
     tm = first + in % rows;
     // (c) `stagger`: column groups that run at the same time on different XCDs start their walk
-    // over the columns at different places, an eighth of the way round per group position.
+    // over the columns at different places, one `xcds`-th of the way round per group position.
     // Otherwise all XCDs miss on the same B panel at the same moment and every miss goes to HBM;
     // staggered, the panel one XCD reads now was read by its neighbour a round of tiles ago and
     // comes from the last-level cache -- provided a round is short enough for it to still be
@@ -503,7 +504,7 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &t
     // 234 -> 199 us; a batch of three K = 8192 / 16384 products 494 -> 517 us.
     const int groups = (tiles_m + GROUP_M - 1) / GROUP_M;
     tn = in / rows;
-    if (stagger) tn = (tn + (group * 8 / groups) * tiles_n / 8) % tiles_n;
+    if (stagger) tn = (tn + (group * xcds / groups) * tiles_n / xcds) % tiles_n;
 }
 
 // Host-side launch helpers shared by the GEMM translation units (defined in mx_gemm.hip).
