@@ -311,6 +311,72 @@ int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t lda, int64
                         int64_t M, void *dw, int dw_dtype, int64_t stride_dwe, int64_t lddw, int64_t N,
                         int64_t Kout, void *stream);
 
+/* ---- expert dispatch either side of the routed-expert GEMMs ------------------------------ */
+
+/*
+ * counts (num_buckets,) int32 [b] = number of i < n with flat_idx[i] == b.  flat_idx holds n
+ * indices of idx_bytes (4: int32, 8: int64) each; values outside [0, num_buckets) are not
+ * counted.  counts is overwritten (it need not be zeroed).  num_buckets <= 8192.
+ * Replaces expert_counts (src/kohakuwullm/models/components/moe.py:38-46), a scatter_add of
+ * ones.
+ */
+int mx_expert_counts(const void *flat_idx, int idx_bytes, int64_t n, int64_t num_buckets, int32_t *counts,
+                     void *stream);
+
+/*
+ * Group the n = T * top_k (token, slot) pairs by expert, given their histogram `counts`
+ * (what mx_expert_counts returns for flat_expert):
+ *   offsets (num_buckets + 1,) = [0, cumsum(counts)];
+ *   order (n,): sorted position -> pair index;  token_of (n,) = order / top_k;
+ *   max_rows (1,) = max(counts) (a diagnostic; may be NULL).
+ * Pairs of one expert keep their input order (a stable sort), so the result is the one of the
+ * reference's sort-based form expert_sort_reference (moe_dispatch.py:264-282) bit for bit and
+ * does not change from run to run; the reference's device path (_expert_offsets :14-37,
+ * _place_pairs :40-57, expert_sort :223-261) leaves the order inside an expert to an atomic
+ * cursor.  Pairs whose expert is outside [0, num_buckets) are left out; positions that a
+ * histogram inconsistent with flat_expert would put outside [0, n) are not written.
+ * workspace: int32 scratch of at least mx_expert_sort_workspace(n, num_buckets) elements,
+ * provided by the caller (nothing is allocated here).  num_buckets <= 1024.
+ */
+int64_t mx_expert_sort_workspace(int64_t n, int64_t num_buckets);
+int mx_expert_sort(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
+                   int64_t num_buckets, int32_t *offsets, int32_t *order, int32_t *token_of, int32_t *max_rows,
+                   int32_t *workspace, int64_t workspace_len, void *stream);
+
+/*
+ * out (num_tokens, d)[t] = sum over the sorted positions p < valid_rows[0] with
+ * order[p] / top_k == t of round(rows[p] * weight[order[p]]): the gated combine of the expert
+ * outputs.  rows (n, d) and out have `dtype` (MX_BF16 / MX_FP16 / MX_FP32), weight
+ * (num_tokens * top_k,) has w_dtype and is indexed by pair; order (n,) holds distinct pair
+ * indices token * top_k + slot (what mx_expert_sort writes; n <= num_tokens * top_k, a pair
+ * that appears nowhere adds nothing).  valid_rows
+ * is a one-element device int32 or NULL (every row counts).  The product is rounded to
+ * `dtype`, the rows of a token are added in ascending sorted position and the sum is rounded
+ * to `dtype` after every addition: the arithmetic of an index_add over the sorted rows
+ * (combine_routed_reference, moe_dispatch.py:203-220), which the reference's device path
+ * (_combine_fwd :60-90, _Combine.forward :134-146) performs with atomic adds in an order that
+ * changes from run to run.  One writer per output element, every element written (out need
+ * not be zeroed).  inv: caller-provided scratch of num_tokens * top_k int32.  d % 8 == 0,
+ * 16-byte aligned rows.
+ */
+int mx_combine_routed(const void *rows, int dtype, int64_t ld, const void *weight, int w_dtype,
+                      const int32_t *order, const int32_t *valid_rows, int32_t *inv, int64_t n, int64_t d,
+                      int64_t num_tokens, int64_t top_k, void *out, int64_t ldo, void *stream);
+
+/*
+ * Both gradients of the combine: for p < valid_rows[0]
+ *   grad_rows[p] = round(grad_out[token_of[p]] * weight[order[p]])       (dtype)
+ *   grad_weight[order[p]] = grad_out[token_of[p]] . rows[p]              (fp32)
+ * and grad_rows[p] = 0 for the other rows; grad_weight (pairs,) fp32 is zeroed first.
+ * Replaces _combine_bwd / _Combine.backward (moe_dispatch.py:93-131, 148-168); the dot
+ * product is one fixed-order fp32 reduction per row instead of atomics over column blocks.
+ */
+int mx_combine_routed_backward(const void *grad_out, int64_t ldg, const void *rows, int64_t ld, int dtype,
+                               const void *weight, int w_dtype, const int32_t *order, const int32_t *token_of,
+                               const int32_t *valid_rows, int64_t n, int64_t d, int64_t num_tokens, int64_t pairs,
+                               void *grad_rows, int64_t ldgr, float *grad_weight, void *stream);
+
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,6 +54,12 @@ SIGNATURES = {
         _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, ctypes.c_float, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
     "mx_rmsnorm_backward": (
         _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
+    "mx_expert_counts": (_ci, [_p, _ci, _i64, _i64, _p, _p]),
+    "mx_expert_sort_workspace": (_i64, [_i64, _i64]),
+    "mx_expert_sort": (_ci, [_p, _ci, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _p]),
+    "mx_combine_routed": (_ci, [_p, _ci, _i64, _p, _ci, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p]),
+    "mx_combine_routed_backward": (
+        _ci, [_p, _i64, _p, _i64, _ci, _p, _ci, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _p]),
     "mx_swizzle_scales": (_ci, [_p, _i64, _i64, _i64, _p, _p]),
     "mx_unswizzle_scales": (_ci, [_p, _i64, _i64, _p, _i64, _p]),
     "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),

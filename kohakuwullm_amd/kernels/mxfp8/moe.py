@@ -16,6 +16,7 @@ from __future__ import annotations
 import torch
 
 from kohakuwullm_amd import _lib
+from kohakuwullm_amd.kernels.moe.moe_dispatch import combine_routed
 from kohakuwullm_amd.kernels.mxfp8.grouped import (
     grouped_mxfp8_gemm,
     grouped_mxfp8_wgrad,
@@ -329,16 +330,6 @@ def _maybe_zeros(sentinel: bool, rows: int, cols: int, like: torch.Tensor):
     if not sentinel:
         return None
     return torch.zeros(rows, cols, device=like.device, dtype=like.dtype)
-
-
-def combine_routed(out_sorted, gate, order, token_of, num_tokens: int, valid_rows=None) -> torch.Tensor:
-    """``out[token_of[m]] += gate[order[m]] * out_sorted[m]`` (``kernels/moe/moe_dispatch.py:264-282`` semantics)."""
-    scaled = out_sorted * gate.index_select(0, order.long()).to(out_sorted.dtype).unsqueeze(1)
-    if valid_rows is not None:
-        keep = torch.arange(out_sorted.shape[0], device=out_sorted.device) < valid_rows
-        scaled = torch.where(keep.unsqueeze(1), scaled, torch.zeros_like(scaled))
-    out = torch.zeros(num_tokens, out_sorted.shape[1], device=out_sorted.device, dtype=out_sorted.dtype)
-    return out.index_add(0, token_of.long(), scaled)
 
 
 def mxfp8_moe_experts_unfused(x, w_in, w_out, gate, token_of, order, offsets, packed: MXFP8ExpertWeights,

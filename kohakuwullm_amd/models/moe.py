@@ -5,9 +5,9 @@ Host-side counterpart of the MXFP8 hooks of the reference's ``MoEMLP``
 ``w_in (E, 2H, dim)`` / ``w_out (E, dim, H)``, the ``mxfp8_matmul`` / ``enable_mxfp8``
 declaration protocol, ``refresh_quantized_weight`` installed on the instance, the cache drop
 on ``_apply``, and the two routed paths (``mxfp8_expert_path`` ``"fused"`` | ``"unfused"``).
-The router and the dispatch here are plain PyTorch: they produce the inputs of the path
-(``offsets``, ``order``, ``token_of`` in the format of
-``src/kohakuwullm/kernels/moe/moe_dispatch.py:223-282``) and are not part of it.
+The router is plain PyTorch; the dispatch (``expert_counts``, ``expert_sort``: ``offsets``,
+``order``, ``token_of`` in the format of ``src/kohakuwullm/kernels/moe/moe_dispatch.py:223-282``)
+and the combine of the unfused path run on the HIP kernels of ``kernels/moe/moe_dispatch.py``.
 """
 
 from __future__ import annotations
@@ -15,6 +15,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from kohakuwullm_amd.kernels.moe.moe_dispatch import expert_counts, expert_sort
 from kohakuwullm_amd.kernels.mxfp8.linear import compute_dtype
 from kohakuwullm_amd.kernels.mxfp8.moe import (
     MXFP8ExpertWeights,
@@ -25,26 +26,6 @@ from kohakuwullm_amd.kernels.mxfp8.moe import (
 from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE
 from kohakuwullm_amd.models.mxfp8_swap import Matmul
 from kohakuwullm_amd.registry import MOE
-
-
-def expert_counts(flat_idx: torch.Tensor, num_buckets: int) -> torch.Tensor:
-    """``(num_buckets,)`` int32 rows per bucket from a flat ``(T * slots,)`` index, without a host sync."""
-    counts = torch.zeros(num_buckets, dtype=torch.int32, device=flat_idx.device)
-    counts.scatter_add_(0, flat_idx.long(), torch.ones_like(flat_idx, dtype=torch.int32))
-    return counts
-
-
-def expert_sort(flat_expert: torch.Tensor, counts: torch.Tensor, top_k: int, num_buckets: int):
-    """Group (token, slot) pairs by expert: ``(offsets (B+1,), order (M,), token_of (M,), counts)``, all int32.
-
-    Stable argsort + cumsum, entirely on the device.  ``order[p]`` is the pair index at sorted
-    position ``p``; ``token_of = order // top_k``.
-    """
-    order = torch.argsort(flat_expert, stable=True).to(torch.int32)
-    offsets = torch.zeros(num_buckets + 1, dtype=torch.int32, device=flat_expert.device)
-    offsets[1:] = torch.cumsum(counts, 0)
-    token_of = torch.div(order, top_k, rounding_mode="floor").to(torch.int32)
-    return offsets, order, token_of, counts
 
 
 class TopKRouter(nn.Module):

@@ -16,6 +16,8 @@ Reference lines followed (paths relative to the reference tree):
   ``src/kohakuwullm/kernels/mxfp8/moe.py:408-433``
 * error metrics ........... ``src/kohakuwullm/bench/core/timing.py:201-228``
 * expert sort (CPU) ....... ``src/kohakuwullm/kernels/moe/moe_dispatch.py:264-282``
+* expert counts, combine .. ``src/kohakuwullm/models/components/moe.py:38-46``,
+  ``src/kohakuwullm/kernels/moe/moe_dispatch.py:60-131,203-220``
 * RMSNorm -> MXFP8 ........ ``src/kohakuwullm/kernels/elementwise/rmsnorm.py:20-128``,
   ``src/kohakuwullm/kernels/mxfp8/fused_act.py:104-143``
 
@@ -249,6 +251,56 @@ def expert_sort(flat_expert: torch.Tensor, num_experts: int, top_k: int):
     offsets = torch.zeros(num_experts + 1, dtype=torch.int32)
     offsets[1:] = counts.cumsum(0).to(torch.int32)
     return offsets, order, (order // top_k).to(torch.int32)
+
+
+def expert_counts(flat_idx: torch.Tensor, num_buckets: int) -> torch.Tensor:
+    """``(num_buckets,)`` int32 histogram of the picks (models/components/moe.py:38-46, a scatter_add of ones)."""
+    return torch.bincount(flat_idx.long(), minlength=num_buckets)[:num_buckets].to(torch.int32)
+
+
+def combine_routed(rows: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, token_of: torch.Tensor,
+                   num_tokens: int, valid_rows: int | None = None) -> torch.Tensor:
+    """``out[token_of[p]] += rows[p] * weight[order[p]]`` over the sorted rows (moe_dispatch.py:203-220).
+
+    The product is taken in fp32 and rounded to ``rows.dtype`` (``_combine_fwd`` :85-88); the
+    additions run in ascending sorted position with the sum rounded to ``rows.dtype`` after each,
+    which is what an ``index_add`` into a 16-bit tensor does.  Written as one vectorized step per
+    "n-th row of its token" so that it does not lean on the loop order inside ``index_add``.
+    """
+    n = rows.shape[0]
+    scaled = (rows.float() * weight.float()[order.long()][:, None]).to(rows.dtype)
+    keep = torch.arange(n) < (n if valid_rows is None else int(valid_rows))
+    tok = token_of.long()
+    out = torch.zeros(num_tokens, rows.shape[1], dtype=rows.dtype)
+    # nth[p] = how many kept rows of the same token sit at lower sorted positions
+    nth = torch.zeros(n, dtype=torch.long)
+    seen = torch.zeros(num_tokens, dtype=torch.long)
+    for p in torch.nonzero(keep).flatten().tolist():
+        nth[p] = seen[tok[p]]
+        seen[tok[p]] += 1
+    for r in range(int(seen.max()) if n else 0):
+        sel = keep & (nth == r)
+        out[tok[sel]] = (out[tok[sel]].float() + scaled[sel].float()).to(rows.dtype)
+    return out
+
+
+def combine_routed_grads(grad_out: torch.Tensor, rows: torch.Tensor, weight: torch.Tensor, order: torch.Tensor,
+                         token_of: torch.Tensor, valid_rows: int | None = None):
+    """``(grad_rows, grad_weight)`` of the combine (``_combine_bwd``, moe_dispatch.py:93-131).
+
+    ``grad_rows`` in ``rows.dtype`` (one fp32 product, one rounding: exact), ``grad_weight`` per
+    pair in fp64 (the kernel sums in fp32; compare with a tolerance).
+    """
+    n = rows.shape[0]
+    keep = torch.arange(n) < (n if valid_rows is None else int(valid_rows))
+    g = grad_out[token_of.long()]
+    grad_rows = (g.float() * weight.float()[order.long()][:, None]).to(rows.dtype)
+    grad_rows[~keep] = 0
+    dots = (g.double() * rows.double()).sum(dim=1)
+    dots[~keep] = 0
+    grad_weight = torch.zeros(weight.numel(), dtype=torch.float64)
+    grad_weight[order.long()] = dots
+    return grad_rows, grad_weight
 
 
 def silu(x: torch.Tensor) -> torch.Tensor:

@@ -16,7 +16,7 @@ def _declared():
     text = open(os.path.join(ROOT, "include", "mxfp8_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     decls = {}
-    for m in re.finditer(r"\b(?:int|const char \*)\s*(mx_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+    for m in re.finditer(r"\b(?:int|int64_t|const char \*)\s*(mx_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
         params = m.group(2).strip()
         decls[m.group(1)] = 0 if params in ("", "void") else params.count(",") + 1
     return decls
@@ -27,7 +27,9 @@ def test_header_parses_to_the_expected_surface():
     assert {"mx_quantize_rows", "mx_quantize_cols", "mx_quantize_dual", "mx_gemm_nt", "mx_grouped_gemm_nt",
             "mx_experts_gemm1", "mx_experts_scatter_gemm", "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt",
             "mx_quantize_cols_grouped", "mx_swiglu_quantize_rows", "mx_swiglu_quantize_dual",
-            "mx_swiglu_bwd_quantize_dual", "mx_abi_version", "mx_strerror", "mx_device_supported"} <= names
+            "mx_swiglu_bwd_quantize_dual", "mx_abi_version", "mx_strerror", "mx_device_supported",
+            "mx_rmsnorm_quantize", "mx_rmsnorm_backward", "mx_expert_counts", "mx_expert_sort_workspace",
+            "mx_expert_sort", "mx_combine_routed", "mx_combine_routed_backward"} <= names
 
 
 def test_library_exports_every_declared_symbol():
@@ -64,3 +66,14 @@ def test_entry_points_validate_before_launch():
     assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 32, 2, 64, 2, 4, 0, None) == _lib.MX_EINVAL  # lda < K
     assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 64, 64, 2, 64, 2, 4, 0, None) == _lib.MX_OK
     assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 64, 2, 64, 2, 4, 1, None) == _lib.MX_EINVAL  # accumulate needs fp32
+    # expert dispatch: sizes, index widths and the workspace are checked before anything is launched
+    assert lib.mx_expert_counts(None, 3, 8, 4, None, None) == _lib.MX_EINVAL  # idx_bytes
+    assert lib.mx_expert_counts(None, 8, 8, 4, None, None) == _lib.MX_EINVAL  # null pointers
+    assert lib.mx_expert_sort_workspace(98304, 64) == 384 * 64 and lib.mx_expert_sort_workspace(0, 5) == 5
+    assert lib.mx_expert_sort_workspace(64 * 4096 * 5, 2) == 4096 * 2 and lib.mx_expert_sort_workspace(-1, 4) == -1
+    assert lib.mx_expert_sort(None, 8, 16, None, 2, 4, None, None, None, None, None, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_combine_routed(None, 0, 16, None, 2, None, None, None, 12, 16, 5, 2, None, 16, None) == _lib.MX_EINVAL  # 12 rows > 5 * 2 pairs
+    assert lib.mx_combine_routed(None, 0, 8, None, 2, None, None, None, 12, 16, 6, 2, None, 16, None) == _lib.MX_EINVAL  # ld < d
+    assert lib.mx_combine_routed(None, 0, 16, None, 2, None, None, None, 0, 16, 0, 2, None, 16, None) == _lib.MX_OK  # empty
+    assert lib.mx_combine_routed_backward(None, 16, None, 16, 3, None, 2, None, None, None, 4, 16, 2, 4, None, 16, None, None) == _lib.MX_EINVAL
+    assert lib.mx_combine_routed_backward(None, 16, None, 16, 0, None, 2, None, None, None, 0, 16, 2, 0, None, 16, None, None) == _lib.MX_OK
