@@ -300,7 +300,38 @@ def build_workload(name: str, dev):
             x.grad = w.grad = None
 
         return step, 0.0, "RMSNorm -> (bf16 out, MXFP8 pair) fwd + bwd on the 32768 x 2048 hidden states of BASELINE configs[2]", lambda: None
+    if name == "dispatch":
+        from kohakuwullm_amd.kernels.moe import combine_routed, expert_counts, expert_sort
+
+        tokens, dim, experts, top_k = 16384, 1024, 64, 6  # the routing of BASELINE configs[3]
+        _, _, _, gate_h, dout_h, offsets_h, order_h, _, _ = make_moe_inputs(tokens, dim, 512, experts, top_k)
+        expert_of_position = torch.repeat_interleave(torch.arange(experts), (offsets_h[1:] - offsets_h[:-1]).long())
+        flat_h = torch.empty(tokens * top_k, dtype=torch.int64)
+        flat_h[order_h.long()] = expert_of_position  # the router's pick of every (token, slot) pair
+        g = torch.Generator().manual_seed(SEED)
+        rows_h = torch.randn(tokens * top_k, dim, generator=g).bfloat16()
+        flat = flat_h.to(dev)
+        rows = [rows_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
+        douts = [dout_h.to(dev) for _ in range(ncopies)]
+        gate = gate_h.float().to(dev).requires_grad_(True)
+
+        def step(i):
+            r = rows[i % ncopies]
+            offsets, order, token_of, _ = expert_sort(flat, expert_counts(flat, experts), top_k, experts)
+            out = combine_routed(r, gate, order, token_of, tokens)
+            out.backward(douts[i % ncopies])
+            r.grad = gate.grad = None
+
+        return step, 0.0, ("expert dispatch of BASELINE configs[3] (16384 tokens, top-6 of 64 experts, 1024 wide): "
+                           "counts + sort + gated combine fwd + bwd"), lambda: None
     raise SystemExit(f"unknown workload {name!r}")
+
+
+# metric and arithmetic type of the workloads that launch streaming kernels only
+STREAM_METRICS = {
+    "norm": ("RMSNorm -> MXFP8 producer fwd+bwd GB/s", "f32 arithmetic on bf16, fp64 sum of squares"),
+    "dispatch": ("expert dispatch (counts, sort, combine fwd+bwd) GB/s", "int32 indices, f32 arithmetic on bf16 rows"),
+}
 
 
 def main() -> None:
@@ -308,7 +339,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm"),
+    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch"),
                     help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
@@ -376,9 +407,9 @@ def main() -> None:
         # a workload of streaming kernels only: the figure of merit is bytes per second against HBM
         step_bytes = quant_bytes / args.steps
         print(json.dumps({
-            "metric": "RMSNorm -> MXFP8 producer fwd+bwd GB/s", "value": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "metric": STREAM_METRICS[args.workload][0], "value": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
             "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 arithmetic on bf16, fp64 sum of squares",
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": STREAM_METRICS[args.workload][1],
             "data": "synthetic", "config": {"workload": desc, "bytes_per_step": int(step_bytes)},
             "roofline": {"kernel": ", ".join(sorted({n for n, _, _ in quant})), "bound": "hbm", "achieved": round(quant_gbs, 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": None,

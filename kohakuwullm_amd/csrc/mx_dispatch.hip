@@ -200,6 +200,19 @@ __device__ __forceinline__ float round_to(float v) {
     return v;
 }
 
+// Two values at once: bf16 goes through the hardware pair conversion (round to nearest even).
+template <int DT>
+__device__ __forceinline__ void round_pair_to(float &a, float &b) {
+    if (DT == MX_BF16) {
+        const uint32_t w = pack2_bf16(settled(a), settled(b));
+        a = bits2f(w << 16);
+        b = bits2f(w & 0xFFFF0000u);
+    } else {
+        a = round_to<DT>(a);
+        b = round_to<DT>(b);
+    }
+}
+
 template <int DT>
 __device__ __forceinline__ void store_row8(void *p, const float (&y)[8]) {
     if (DT == MX_FP32) {
@@ -222,13 +235,32 @@ __device__ __forceinline__ float load_weight(const void *w, int64_t i) {
     return Elem<WDT>::load1((const typename Elem<WDT>::type *)w + i);
 }
 
+// One thread per token: its top_k entries of inv in ascending order, absent pairs (-1) last.
+__global__ __launch_bounds__(256) void combine_sort_kernel(int32_t *__restrict__ inv, int top_k, int64_t tokens) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= tokens) return;
+    int32_t *mine = inv + t * top_k;
+    for (int i = 1; i < top_k; i++) {
+        const int32_t v = mine[i];
+        const uint32_t key = (uint32_t)v;  // -1 compares as the largest
+        int j = i - 1;
+        while (j >= 0 && (uint32_t)mine[j] > key) {
+            mine[j + 1] = mine[j];
+            j--;
+        }
+        mine[j + 1] = v;
+    }
+}
+
 // One thread per 8 columns of a token.  The token's rows are added in ascending sorted position
-// (the order of an index_add over the sorted rows); the product and every partial sum are
-// rounded to the row type, as a 16-bit accumulator in memory would.
+// (the order of an index_add over the sorted rows; `sorted` holds them in that order); the
+// product and every partial sum are rounded to the row type, as a 16-bit accumulator in memory
+// would.  Rows are fetched four at a time so that their loads overlap.
 template <int DT, int WDT>
 __global__ __launch_bounds__(256) void combine_routed_kernel(const void *__restrict__ rows, int64_t ld,
                                                               const void *__restrict__ weight,
-                                                              const int32_t *__restrict__ inv, int top_k,
+                                                              const int32_t *__restrict__ order,
+                                                              const int32_t *__restrict__ sorted, int top_k,
                                                               void *__restrict__ out, int64_t ldo, int64_t tokens,
                                                               int d8) {
 #pragma clang fp contract(off)  // fp32 rows: the product is rounded before it is added, never fused
@@ -240,21 +272,30 @@ __global__ __launch_bounds__(256) void combine_routed_kernel(const void *__restr
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) acc[e] = 0.0f;
-    const int32_t *mine = inv + t * top_k;
-    int last = -1;
-    for (int k = 0; k < top_k; k++) {
-        int pos = 0x7FFFFFFF, slot = 0;
-        for (int j = 0; j < top_k; j++) {
-            const int p = mine[j];
-            if (p > last && p < pos) pos = p, slot = j;
-        }
-        if (pos == 0x7FFFFFFF) break;
-        last = pos;
-        const float scale = load_weight<WDT>(weight, t * top_k + slot);
-        float v[8];
-        Elem<DT>::load8((const T *)rows + (int64_t)pos * ld + col, v);
+    const int32_t *mine = sorted + t * top_k;
+    for (int k0 = 0; k0 < top_k; k0 += 4) {
+        int pos[4];
+        float scale[4], v[4][8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] = round_to<DT>(acc[e] + round_to<DT>(v[e] * scale));
+        for (int u = 0; u < 4; u++) pos[u] = k0 + u < top_k ? mine[k0 + u] : -1;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (pos[u] < 0) continue;
+            scale[u] = load_weight<WDT>(weight, order[pos[u]]);
+            Elem<DT>::load8((const T *)rows + (int64_t)pos[u] * ld + col, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (pos[u] < 0) continue;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                float a = v[u][e] * scale[u], b = v[u][e + 1] * scale[u];
+                round_pair_to<DT>(a, b);
+                a += acc[e], b += acc[e + 1];
+                round_pair_to<DT>(a, b);
+                acc[e] = a, acc[e + 1] = b;
+            }
+        }
     }
     store_row8<DT>((T *)out + t * ldo + col, acc);
 }
@@ -313,12 +354,13 @@ static int sort_rounds(int64_t n) {
 }
 
 template <int DT>
-static int launch_combine(int w_dtype, const void *rows, int64_t ld, const void *weight, const int32_t *inv, int top_k,
-                          void *out, int64_t ldo, int64_t tokens, int d8, unsigned blocks, hipStream_t st) {
+static int launch_combine(int w_dtype, const void *rows, int64_t ld, const void *weight, const int32_t *order,
+                          const int32_t *inv, int top_k, void *out, int64_t ldo, int64_t tokens, int d8, unsigned blocks,
+                          hipStream_t st) {
     switch (w_dtype) {
-    case MX_BF16: combine_routed_kernel<DT, MX_BF16><<<dim3(blocks), dim3(256), 0, st>>>(rows, ld, weight, inv, top_k, out, ldo, tokens, d8); break;
-    case MX_FP16: combine_routed_kernel<DT, MX_FP16><<<dim3(blocks), dim3(256), 0, st>>>(rows, ld, weight, inv, top_k, out, ldo, tokens, d8); break;
-    default: combine_routed_kernel<DT, MX_FP32><<<dim3(blocks), dim3(256), 0, st>>>(rows, ld, weight, inv, top_k, out, ldo, tokens, d8); break;
+    case MX_BF16: combine_routed_kernel<DT, MX_BF16><<<dim3(blocks), dim3(256), 0, st>>>(rows, ld, weight, order, inv, top_k, out, ldo, tokens, d8); break;
+    case MX_FP16: combine_routed_kernel<DT, MX_FP16><<<dim3(blocks), dim3(256), 0, st>>>(rows, ld, weight, order, inv, top_k, out, ldo, tokens, d8); break;
+    default: combine_routed_kernel<DT, MX_FP32><<<dim3(blocks), dim3(256), 0, st>>>(rows, ld, weight, order, inv, top_k, out, ldo, tokens, d8); break;
     }
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
@@ -353,7 +395,7 @@ extern "C" int mx_expert_counts(const void *flat_idx, int idx_bytes, int64_t n, 
     hipStream_t st = (hipStream_t)stream;
     dispatch_fill_kernel<<<dim3((unsigned)((num_buckets + 255) / 256)), dim3(256), 0, st>>>(counts, num_buckets, 0);
     if (n) {
-        const int64_t per_block = 4096;
+        const int64_t per_block = 1024;
         const dim3 grid((unsigned)((n + per_block - 1) / per_block)), block(256);
         const size_t lds = (size_t)num_buckets * sizeof(int32_t);
         if (idx_bytes == 8)
@@ -410,10 +452,11 @@ extern "C" int mx_combine_routed(const void *rows, int dtype, int64_t ld, const 
     hipStream_t st = (hipStream_t)stream;
     dispatch_fill_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>(inv, pairs, -1);
     if (n) combine_invert_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(order, valid_rows, n, pairs, inv);
+    if (n && top_k > 1) combine_sort_kernel<<<dim3((unsigned)((num_tokens + 255) / 256)), dim3(256), 0, st>>>(inv, (int)top_k, num_tokens);
     switch (dtype) {
-    case MX_BF16: return launch_combine<MX_BF16>(w_dtype, rows, ld, weight, inv, (int)top_k, out, ldo, num_tokens, (int)(d / 8), (unsigned)blocks, st);
-    case MX_FP16: return launch_combine<MX_FP16>(w_dtype, rows, ld, weight, inv, (int)top_k, out, ldo, num_tokens, (int)(d / 8), (unsigned)blocks, st);
-    default: return launch_combine<MX_FP32>(w_dtype, rows, ld, weight, inv, (int)top_k, out, ldo, num_tokens, (int)(d / 8), (unsigned)blocks, st);
+    case MX_BF16: return launch_combine<MX_BF16>(w_dtype, rows, ld, weight, order, inv, (int)top_k, out, ldo, num_tokens, (int)(d / 8), (unsigned)blocks, st);
+    case MX_FP16: return launch_combine<MX_FP16>(w_dtype, rows, ld, weight, order, inv, (int)top_k, out, ldo, num_tokens, (int)(d / 8), (unsigned)blocks, st);
+    default: return launch_combine<MX_FP32>(w_dtype, rows, ld, weight, order, inv, (int)top_k, out, ldo, num_tokens, (int)(d / 8), (unsigned)blocks, st);
     }
 }
 

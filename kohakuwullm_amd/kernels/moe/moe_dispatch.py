@@ -110,7 +110,7 @@ class _Combine(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         grad_rows = torch.empty_like(rows)
         grad_weight = torch.empty(weight.numel(), dtype=torch.float32, device=rows.device)
-        _lib.invoke("mx_combine_routed_backward", rows.element_size() * dim * 3 * n, rows,
+        _lib.invoke("mx_combine_routed_backward", rows.element_size() * dim * (2 * n + grad_out.shape[0]), rows,
                     grad_out.data_ptr(), grad_out.stride(0), rows.data_ptr(), rows.stride(0), _lib.MX_DTYPE[rows.dtype],
                     weight.data_ptr(), _lib.MX_DTYPE[weight.dtype], order.data_ptr(), token_of.data_ptr(),
                     _valid_ptr(valid_rows, rows.device), n, dim, grad_out.shape[0], weight.numel(),
