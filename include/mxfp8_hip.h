@@ -91,6 +91,23 @@ int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t l
                      uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
 
 /*
+ * mx_quantize_dual of `count` matrices behind one launch (one per 24 of them): the
+ * once-per-optimizer-step requantization of every weight matrix of a model, which the
+ * reference performs as one launch per matrix and axis from refresh_mxfp8_weights
+ * (src/kohakuwullm/models/mxfp8_swap.py:331-343; MXFP8Linear.refresh_quantized_weight,
+ * src/kohakuwullm/kernels/mxfp8/linear.py:98-108; MXFP8ExpertWeights.refresh,
+ * src/kohakuwullm/kernels/mxfp8/moe.py:34-61).  Every problem has the arguments of
+ * mx_quantize_dual and gets the same bytes; all are validated before anything is launched.
+ */
+typedef struct {
+    const void *x;      /* (M,K), row pitch ldx elements, dtype x_dtype */
+    uint8_t *q, *s;     /* (M,K) codes and (M,K/32) scale bytes, blocks along K */
+    uint8_t *qT, *sT;   /* (K,M) codes and (K,M/32) scale bytes, blocks along M */
+    int64_t M, K, ldx, ldq, lds, ldqT, ldsT;
+} mx_quant_problem;
+int mx_quantize_dual_batch(const mx_quant_problem *problems, int count, int x_dtype, void *stream);
+
+/*
  * q,s = quantize_rows(silu(gate) * up) with the product kept in fp32.
  * gate, up (M,K) unit inner stride, row pitches ldg, ldu.  K % 32 == 0.
  * Replaces swiglu_mx / _swiglu_mx_kernel (src/kohakuwullm/kernels/mxfp8/fused_act.py:17-101).

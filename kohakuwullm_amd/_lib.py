@@ -30,6 +30,7 @@ SIGNATURES = {
     "mx_quantize_rows": (_ci, [_p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_quantize_cols": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_quantize_dual_batch": (_ci, [_p, _ci, _ci, _p]),
     "mx_swiglu_quantize_rows": (_ci, [_p, _p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_swiglu_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
     "mx_swiglu_bwd_quantize_dual": (
@@ -73,6 +74,16 @@ class GemmProblem(ctypes.Structure):
     _fields_ = [(n, _p) for n in ("aq", "a_scale", "bq", "b_scale", "c")] + [
         (n, _i64) for n in ("M", "N", "K", "lda", "ldas", "ldb", "ldbs", "ldc")
     ]
+
+
+
+class QuantProblem(ctypes.Structure):
+    """``mx_quant_problem`` of the C header."""
+
+    _fields_ = [(n, _p) for n in ("x", "q", "s", "qT", "sT")] + [
+        (n, _i64) for n in ("M", "K", "ldx", "ldq", "lds", "ldqT", "ldsT")
+    ]
+
 
 _lib: ctypes.CDLL | None = None
 

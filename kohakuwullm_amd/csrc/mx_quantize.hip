@@ -248,6 +248,48 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict_
     quant_tile<DUAL>(v, o, M, K, m0, k0, tile, tscale);
 }
 
+// Several matrices behind one launch: workgroup `id` finds its matrix in the running tile
+// totals and quantizes one 128 x 128 tile of it along both axes.  For the once-per-step
+// requantization of all weight matrices of a model, where a launch per matrix (and per axis)
+// costs more than the bytes it moves.
+#define MX_QUANT_BATCH_MAX 24
+struct QuantBatchArgs {
+    const void *x[MX_QUANT_BATCH_MAX];
+    int64_t M[MX_QUANT_BATCH_MAX], K[MX_QUANT_BATCH_MAX], ldx[MX_QUANT_BATCH_MAX];
+    QuantTileOut o[MX_QUANT_BATCH_MAX];
+    int tile_end[MX_QUANT_BATCH_MAX];  // tiles of problems 0..j
+    int tiles_k[MX_QUANT_BATCH_MAX];
+    int count;
+};
+
+template <int DT>
+__global__ __launch_bounds__(256) void quant_dual_batch_kernel(QuantBatchArgs b) {
+    typedef typename Elem<DT>::type T;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QC_TILE * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
+    const int t = threadIdx.x;
+    int j = 0;
+    while (j + 1 < b.count && (int)blockIdx.x >= b.tile_end[j]) j++;
+    const int local = (int)blockIdx.x - (j ? b.tile_end[j - 1] : 0);
+    const int64_t M = b.M[j], K = b.K[j], ldx = b.ldx[j];
+    const void *x = b.x[j];
+    const int64_t m0 = (int64_t)(local / b.tiles_k[j]) * QC_TILE, k0 = (int64_t)(local % b.tiles_k[j]) * QC_TILE;
+    const int64_t col = k0 + (t & 15) * 8;
+    const int64_t row0 = m0 + (t >> 4) * 8;
+    const bool ok = col < K && m0 + (t >> 6) * 32 < M;
+    float v[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (ok) {
+            Elem<DT>::load8((const T *)x + (row0 + i) * ldx + col, v[i]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
+        }
+    }
+    quant_tile<true>(v, b.o[j], M, K, m0, k0, tile, tscale);
+}
+
 __device__ __forceinline__ float sigmoid_fast(float x) { return __fdividef(1.0f, 1.0f + __expf(-x)); }
 
 // h = silu(g) * u from the fused projection output gu (M, 2H) (gate half first), quantized
@@ -593,6 +635,58 @@ extern "C" int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K
     case MX_FP32: return launch_cols<MX_FP32, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
     default: return MX_EINVAL;
     }
+}
+
+extern "C" int mx_quantize_dual_batch(const mx_quant_problem *problems, int count, int x_dtype, void *stream) {
+    if (count < 0 || (count > 0 && !problems)) return MX_EINVAL;
+    if (x_dtype != MX_BF16 && x_dtype != MX_FP16 && x_dtype != MX_FP32) return MX_EINVAL;
+    for (int j = 0; j < count; j++) {  // validate everything before launching anything
+        const mx_quant_problem &p = problems[j];
+        if (p.M < 0 || p.K < 0 || p.M % MX_BLOCK || p.K % MX_BLOCK || p.ldx < p.K || p.ldq < p.K ||
+            p.lds < p.K / MX_BLOCK || p.ldqT < p.M || p.ldsT < p.M / MX_BLOCK)
+            return MX_EINVAL;
+        if (p.M && p.K && (!p.x || !p.q || !p.s || !p.qT || !p.sT)) return MX_EINVAL;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    QuantBatchArgs b;
+    b.count = 0;
+    int64_t total = 0;
+    auto flush = [&]() -> int {
+        if (b.count) {
+            const dim3 grid((unsigned)total), block(256);
+            switch (x_dtype) {
+            case MX_BF16: quant_dual_batch_kernel<MX_BF16><<<grid, block, 0, st>>>(b); break;
+            case MX_FP16: quant_dual_batch_kernel<MX_FP16><<<grid, block, 0, st>>>(b); break;
+            default: quant_dual_batch_kernel<MX_FP32><<<grid, block, 0, st>>>(b); break;
+            }
+            MX_LAUNCH_CHECK();
+        }
+        b.count = 0, total = 0;
+        return MX_OK;
+    };
+    for (int j = 0; j < count; j++) {
+        const mx_quant_problem &p = problems[j];
+        if (p.M == 0 || p.K == 0) continue;
+        const int64_t tiles_k = (p.K + QC_TILE - 1) / QC_TILE, tiles = tiles_k * ((p.M + QC_TILE - 1) / QC_TILE);
+        if (!cols_vec_ok(p.x, x_dtype, p.K, p.ldx, p.qT, p.ldqT) || !aligned(p.q, 8) || p.ldq % 8 ||
+            tiles > 0x3FFFFFFF) {
+            // an operand the tiled kernel does not take goes through the single-matrix entry point
+            int rc = mx_quantize_dual(p.x, x_dtype, p.M, p.K, p.ldx, p.q, p.ldq, p.s, p.lds, p.qT, p.ldqT, p.sT, p.ldsT,
+                                      stream);
+            if (rc != MX_OK) return rc;
+            continue;
+        }
+        if (b.count == MX_QUANT_BATCH_MAX || total + tiles > 0x3FFFFFFF) {
+            int rc = flush();
+            if (rc != MX_OK) return rc;
+        }
+        const int k = b.count++;
+        b.x[k] = p.x, b.M[k] = p.M, b.K[k] = p.K, b.ldx[k] = p.ldx;
+        b.o[k] = tile_out(p.qT, p.ldqT, p.sT, p.ldsT, p.q, p.ldq, p.s, p.lds);
+        total += tiles;
+        b.tile_end[k] = (int)total, b.tiles_k[k] = (int)tiles_k;
+    }
+    return flush();
 }
 
 template <int DT>

@@ -14,6 +14,7 @@ from kohakuwullm_amd.kernels.mxfp8.quantize import (
     quantize_mx,
     quantize_mx_cols,
     quantize_mx_dual,
+    quantize_mx_dual_batch,
 )
 
 
@@ -34,5 +35,6 @@ __all__ = [
     "quantize_mx",
     "quantize_mx_cols",
     "quantize_mx_dual",
+    "quantize_mx_dual_batch",
     "quantize_mx_vendor",
 ]

@@ -144,6 +144,20 @@ class MXFP8Linear(torch.nn.Module):
             wq_d, ws_d = quantize_mx(self._pad_k(self.weight.t()))
         self._cache = (wq_f, ws_f, wq_d, ws_d)
 
+    def mxfp8_refresh_plan(self) -> list[torch.Tensor] | None:
+        """The matrices whose row + column quantization is this module's cache, for a batched refresh.
+
+        ``None`` when the cache is not a plain dual quantization of the weight (padded
+        ``out_features``); ``refresh_mxfp8_weights`` then calls ``refresh_quantized_weight``.
+        """
+        if self._pad_k.width or self.out_features % BLOCK_SCALE or not self.weight.is_cuda:
+            return None
+        return [self.weight.detach()]
+
+    def mxfp8_install(self, copies) -> None:
+        """Take the ``(q, s, qT, sT)`` a batched refresh made of the planned matrix."""
+        (self._cache,) = copies
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self._cache is None:
             self.refresh_quantized_weight()

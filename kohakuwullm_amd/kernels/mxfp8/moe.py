@@ -61,8 +61,9 @@ class MXFP8ExpertWeights:
 
     __slots__ = ("in_fwd", "in_dgrad", "out_fwd", "out_dgrad")
 
-    def __init__(self, w_in: torch.Tensor, w_out: torch.Tensor) -> None:
-        self.refresh(w_in, w_out)
+    def __init__(self, w_in: torch.Tensor | None = None, w_out: torch.Tensor | None = None) -> None:
+        if w_in is not None:
+            self.refresh(w_in, w_out)
 
     @torch.no_grad()
     def refresh(self, w_in: torch.Tensor, w_out: torch.Tensor) -> None:
@@ -71,6 +72,29 @@ class MXFP8ExpertWeights:
         self.out_fwd = _quantize_stacked(w_out)  # (E, dim, H), K = H
         self.in_dgrad = _quantize_stacked_t(w_in)  # (E, dim, 2H), K = 2H
         self.out_dgrad = _quantize_stacked_t(w_out)  # (E, H, dim), K = dim
+
+    @staticmethod
+    def plan(w_in: torch.Tensor, w_out: torch.Tensor) -> list[torch.Tensor] | None:
+        """The two stacks as ``(E*N, K)`` matrices whose dual quantization holds all four copies.
+
+        ``None`` when a stack cannot be taken as one matrix (rows per expert not a multiple of
+        128, or a non-contiguous stack): ``refresh`` is the way then.
+        """
+        for w in (w_in, w_out):
+            if w.shape[1] % 128 or w.shape[2] % BLOCK_SCALE or not w.is_contiguous() or not w.is_cuda:
+                return None
+        return [w.detach().reshape(w.shape[0] * w.shape[1], w.shape[2]) for w in (w_in, w_out)]
+
+    def install(self, copies, num_experts: int) -> None:
+        """Take the dual quantizations of ``plan``'s matrices, viewed per expert as ``refresh`` lays them out."""
+        views = []
+        for q, s, qt, st in copies:
+            en, k = q.shape
+            n = en // num_experts
+            views.append((q.view(num_experts, n, k), s.view(num_experts, n, k // BLOCK_SCALE)))
+            views.append((qt.view(k, num_experts, n).permute(1, 0, 2),
+                          st.view(k, num_experts, n // BLOCK_SCALE).permute(1, 0, 2)))
+        self.in_fwd, self.in_dgrad, self.out_fwd, self.out_dgrad = views
 
 
 def _w_args(wq, ws):

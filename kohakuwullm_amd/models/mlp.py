@@ -99,6 +99,16 @@ class MXFP8SwiGLU(nn.Module):
             quantize_mx_cols(self.w_out),
         )
 
+    def mxfp8_refresh_plan(self) -> list[torch.Tensor] | None:
+        """Both matrices as dual (row + column axis) quantizations, for ``refresh_mxfp8_weights``' single launch."""
+        if self.dim % 32 or self.hidden % 32 or not self.w_in.is_cuda:
+            return None
+        return [self.w_in.detach(), self.w_out.detach()]
+
+    def mxfp8_install(self, copies) -> None:
+        (q1, s1, qt1, st1), (q2, s2, qt2, st2) = copies
+        self._packed = ((q1, s1), (qt1, st1), (q2, s2), (qt2, st2))
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self._packed is None:
             self.refresh_quantized_weight()

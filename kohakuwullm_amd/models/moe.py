@@ -94,6 +94,17 @@ class MoEMLP(nn.Module):
         else:
             self._packed.refresh(self.w_in, self.w_out)
 
+    def mxfp8_refresh_plan(self):
+        """The expert stacks as two matrices for ``refresh_mxfp8_weights``' single launch (``None``: refresh alone)."""
+        if self._routed == self._routed_eager:
+            return None
+        return MXFP8ExpertWeights.plan(self.w_in, self.w_out)
+
+    def mxfp8_install(self, copies) -> None:
+        if self._packed is None:
+            self._packed = MXFP8ExpertWeights()
+        self._packed.install(copies, self.num_experts)
+
     def _apply(self, *args, **kwargs):
         self._packed = None
         return super()._apply(*args, **kwargs)

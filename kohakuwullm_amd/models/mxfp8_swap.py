@@ -21,6 +21,7 @@ import torch
 import torch.nn as nn
 
 from kohakuwullm_amd.kernels.mxfp8.linear import MXFP8Linear
+from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx_dual_batch
 
 # Declaration protocol for matmul a module holds as bare parameters: the attribute names
 # `swap_mxfp8` looks up, and what `mxfp8_matmul()` returns per tensor.  Field for field the
@@ -204,11 +205,31 @@ def swap_mxfp8(model: nn.Module, linear_cls: type = MXFP8Linear, convert_declare
 
 
 def refresh_mxfp8_weights(model: nn.Module) -> int:
-    """Requantize every MXFP8 weight cache; call after every optimizer step.  Returns the module count."""
+    """Requantize every MXFP8 weight cache; call after every optimizer step.  Returns the module count.
+
+    Same contract as the reference (``src/kohakuwullm/models/mxfp8_swap.py:331-343``); the modules
+    that describe their cache as dual quantizations of whole matrices (``mxfp8_refresh_plan`` /
+    ``mxfp8_install``) are served together, one launch per 24 matrices instead of two launches
+    and four allocations per matrix, the others through their own ``refresh_quantized_weight``.
+    """
     count = 0
+    planned: dict[tuple, list] = {}
     for module in model.modules():
         refresh = getattr(module, "refresh_quantized_weight", None)
-        if callable(refresh):
+        if not callable(refresh):
+            continue
+        count += 1
+        plan_of = getattr(module, "mxfp8_refresh_plan", None)
+        plan = plan_of() if callable(plan_of) else None
+        if not plan:
             refresh()
-            count += 1
+            continue
+        planned.setdefault((plan[0].device, plan[0].dtype), []).append((module, plan))
+    for group in planned.values():
+        with torch.no_grad():
+            copies = quantize_mx_dual_batch([x for _, plan in group for x in plan])
+        at = 0
+        for module, plan in group:
+            module.mxfp8_install(copies[at : at + len(plan)])
+            at += len(plan)
     return count

@@ -77,3 +77,13 @@ def test_entry_points_validate_before_launch():
     assert lib.mx_combine_routed(None, 0, 16, None, 2, None, None, None, 0, 16, 0, 2, None, 16, None) == _lib.MX_OK  # empty
     assert lib.mx_combine_routed_backward(None, 16, None, 16, 3, None, 2, None, None, None, 4, 16, 2, 4, None, 16, None, None) == _lib.MX_EINVAL
     assert lib.mx_combine_routed_backward(None, 16, None, 16, 0, None, 2, None, None, None, 0, 16, 2, 0, None, 16, None, None) == _lib.MX_OK
+    # the batched quantizer validates every problem before it launches anything
+    probs = (_lib.QuantProblem * 2)()
+    probs[0] = _lib.QuantProblem(None, None, None, None, None, 0, 64, 64, 64, 2, 0, 0)
+    probs[1] = _lib.QuantProblem(None, None, None, None, None, 48, 64, 64, 64, 2, 48, 1)  # M % 32
+    assert lib.mx_quantize_dual_batch(ctypes.byref(probs), 1, 0, None) == _lib.MX_OK  # an empty matrix
+    assert lib.mx_quantize_dual_batch(ctypes.byref(probs), 2, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_quantize_dual_batch(None, 1, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_quantize_dual_batch(ctypes.byref(probs), 1, 7, None) == _lib.MX_EINVAL  # dtype
+    probs[1] = _lib.QuantProblem(None, None, None, None, None, 64, 64, 64, 64, 2, 64, 2)  # null operands
+    assert lib.mx_quantize_dual_batch(ctypes.byref(probs), 2, 0, None) == _lib.MX_EINVAL
