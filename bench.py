@@ -324,6 +324,33 @@ def build_workload(name: str, dev):
 
         return step, 0.0, ("expert dispatch of BASELINE configs[3] (16384 tokens, top-6 of 64 experts, 1024 wide): "
                            "counts + sort + gated combine fwd + bwd"), lambda: None
+    if name == "refresh":
+        from kohakuwullm_amd.models.mlp import MXFP8SwiGLU
+        from kohakuwullm_amd.models.mxfp8_swap import refresh_mxfp8_weights
+
+        # every linear weight of a 546M-class dense model: 20 blocks of the feed-forward pair of
+        # BASELINE configs[1] (dim 1536, ffn 4096) and GQA projections of the same width (12 query and
+        # 4 KV heads of 128): 80 matrices, 503 M parameters
+        dim, ffn, blocks = 1536, 4096, 20
+        torch.manual_seed(SEED)
+        model = torch.nn.ModuleList()
+        for _ in range(blocks):
+            model.append(MXFP8Linear(dim, dim + 2 * 512))
+            model.append(MXFP8Linear(dim, dim))
+            model.append(MXFP8SwiGLU(dim, hidden=ffn))
+        model.to(dev)
+        params = sum(p.numel() for p in model.parameters())
+
+        def step(i):
+            refresh_mxfp8_weights(model)
+
+        def one_by_one():
+            for module in model:
+                module.refresh_quantized_weight()
+
+        step.alternative = ("ms_per_step_one_module_at_a_time", one_by_one)
+        return step, 0.0, (f"requantization of all {4 * blocks} linear weights ({params / 1e6:.0f} M parameters, bf16 masters) of a "
+                           "546M-class dense model along both axes: refresh_mxfp8_weights, once per optimizer step"), lambda: None
     raise SystemExit(f"unknown workload {name!r}")
 
 
@@ -331,6 +358,7 @@ def build_workload(name: str, dev):
 STREAM_METRICS = {
     "norm": ("RMSNorm -> MXFP8 producer fwd+bwd GB/s", "f32 arithmetic on bf16, fp64 sum of squares"),
     "dispatch": ("expert dispatch (counts, sort, combine fwd+bwd) GB/s", "int32 indices, f32 arithmetic on bf16 rows"),
+    "refresh": ("MXFP8 weight requantization (row + column axis) GB/s", "bf16 -> e4m3 + ue8m0"),
 }
 
 
@@ -339,7 +367,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch"),
+    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh"),
                     help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
@@ -406,6 +434,17 @@ def main() -> None:
     if not gemm:
         # a workload of streaming kernels only: the figure of merit is bytes per second against HBM
         step_bytes = quant_bytes / args.steps
+        extra = {}
+        if hasattr(step, "alternative"):  # the same work done another way, timed the same way, for comparison
+            key, other = step.alternative
+            for _ in range(args.warmup):
+                other()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                other()
+            torch.cuda.synchronize()
+            extra[key] = round((time.perf_counter() - t0) / args.steps * 1e3, 4)
         print(json.dumps({
             "metric": STREAM_METRICS[args.workload][0], "value": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
             "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -414,6 +453,7 @@ def main() -> None:
             "roofline": {"kernel": ", ".join(sorted({n for n, _, _ in quant})), "bound": "hbm", "achieved": round(quant_gbs, 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": None,
                          "launches": len(quant), "avg_launch_us": round(quant_ms / len(quant) * 1e3, 2)},
+            **extra,
         }))
         return
     gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12

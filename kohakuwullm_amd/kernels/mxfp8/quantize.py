@@ -103,20 +103,13 @@ def quantize_mx_dual(x: torch.Tensor):
     return q, s, qt, st
 
 
-def _carve(arena: torch.Tensor, cursor: int, shape: tuple[int, int], dtype) -> tuple[torch.Tensor, int]:
-    """A ``shape`` view of one-byte elements at ``cursor`` of ``arena``; the next cursor is 256-byte aligned."""
-    size = shape[0] * shape[1]
-    view = arena[cursor : cursor + size].view(dtype).view(shape)
-    return view, cursor + (size + 255) // 256 * 256
-
-
 def quantize_mx_dual_batch(xs: list[torch.Tensor]) -> list[tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]]:
     """``quantize_mx_dual`` of every matrix of ``xs`` behind one launch per 24 matrices.
 
     For the once-per-optimizer-step requantization of a model's weights, where a launch and four
     allocations per matrix cost more than the bytes moved.  The matrices must share device and
-    dtype; the outputs of one call are views of a single allocation.  Same bytes as
-    ``quantize_mx_dual`` on each.
+    dtype; the codes of one call are views of one allocation, the scale bytes of another.  Same
+    bytes as ``quantize_mx_dual`` on each.
     """
     if not xs:
         return []
@@ -127,21 +120,27 @@ def quantize_mx_dual_batch(xs: list[torch.Tensor]) -> list[tuple[torch.Tensor, t
         if x.device != xs[0].device or x.dtype != xs[0].dtype:
             raise ValueError("quantize_mx_dual_batch: the matrices must share one device and one dtype")
     xs = [x if x.stride(1) == 1 else x.contiguous() for x in xs]
-    per = [((m * k + 255) // 256 * 256, (m * k // BLOCK_SCALE + 255) // 256 * 256) for m, k in (x.shape for x in xs)]
-    arena = torch.empty(2 * sum(a + b for a, b in per), device=xs[0].device, dtype=torch.uint8)
+    # sizes are multiples of 1024 (codes) and 32 (scale bytes): every piece starts 16-byte aligned
+    n_codes = [x.shape[0] * x.shape[1] for x in xs]
+    n_scales = [n // BLOCK_SCALE for n in n_codes]
+    codes = torch.empty(2 * sum(n_codes), device=xs[0].device, dtype=_FP8)
+    scales = torch.empty(2 * sum(n_scales), device=xs[0].device, dtype=torch.uint8)
+    code_views = codes.split_with_sizes([n for n in n_codes for _ in (0, 1)])
+    scale_views = scales.split_with_sizes([n for n in n_scales for _ in (0, 1)])
     problems = (_lib.QuantProblem * len(xs))()
-    out, cursor, work = [], 0, 0.0
+    out, at_code, at_scale, work = [], codes.data_ptr(), scales.data_ptr(), 0.0
     for j, x in enumerate(xs):
         m, k = x.shape
-        q, cursor = _carve(arena, cursor, (m, k), _FP8)
-        s, cursor = _carve(arena, cursor, (m, k // BLOCK_SCALE), torch.uint8)
-        qt, cursor = _carve(arena, cursor, (k, m), _FP8)
-        st, cursor = _carve(arena, cursor, (k, m // BLOCK_SCALE), torch.uint8)
-        problems[j] = _lib.QuantProblem(x.data_ptr(), q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
-                                        m, k, x.stride(0), k, k // BLOCK_SCALE, m, m // BLOCK_SCALE)
-        out.append((q, s, qt, st))
-        work += m * k * (x.element_size() + 2 * (1 + 1 / BLOCK_SCALE))
-    _lib.invoke("mx_quantize_dual_batch", work, xs[0], ctypes.byref(problems), len(xs), _lib.MX_DTYPE[xs[0].dtype])
+        kb, mb = k // BLOCK_SCALE, m // BLOCK_SCALE
+        problems[j] = _lib.QuantProblem(x.data_ptr(), at_code, at_scale, at_code + n_codes[j], at_scale + n_scales[j],
+                                        m, k, x.stride(0), k, kb, m, mb)
+        out.append((code_views[2 * j].view(m, k), scale_views[2 * j].view(m, kb),
+                    code_views[2 * j + 1].view(k, m), scale_views[2 * j + 1].view(k, mb)))
+        at_code += 2 * n_codes[j]
+        at_scale += 2 * n_scales[j]
+        work += n_codes[j] * (x.element_size() + 2 * (1 + 1 / BLOCK_SCALE))
+    if codes.numel():
+        _lib.invoke("mx_quantize_dual_batch", work, xs[0], ctypes.byref(problems), len(xs), _lib.MX_DTYPE[xs[0].dtype])
     return out
 
 
