@@ -324,6 +324,23 @@ def build_workload(name: str, dev):
 
         return step, 0.0, ("expert dispatch of BASELINE configs[3] (16384 tokens, top-6 of 64 experts, 1024 wide): "
                            "counts + sort + gated combine fwd + bwd"), lambda: None
+    if name == "heads":
+        from kohakuwullm_amd.kernels.mxfp8.attention_quant import column_mean, quantize_heads
+
+        # q and k of the fused projection output of BASELINE configs[2]: 32768 tokens, 16 query and 4 KV heads of 128
+        tokens, hq, hkv, d = 32768, 16, 4, 128
+        g = torch.Generator().manual_seed(SEED)
+        qkv_h = torch.randn(tokens, (hq + 2 * hkv) * d, generator=g).bfloat16()
+        qkvs = [qkv_h.to(dev) for _ in range(ncopies)]
+        mus = [column_mean(qkvs[0][:, lo : lo + n * d].view(tokens, n, d)) for lo, n in ((0, hq), (hq * d, hkv))]
+
+        def step(i):
+            qkv = qkvs[i % ncopies]
+            quantize_heads(qkv[:, : hq * d].view(tokens, hq, d), mus[0])
+            quantize_heads(qkv[:, hq * d : (hq + hkv) * d].view(tokens, hkv, d), mus[1])
+
+        return step, 0.0, ("MXFP8 QK^T operands: q (16 heads) and k (4 heads) of 128 channels, 32768 tokens, read in place from the "
+                           "fused projection output of BASELINE configs[2], per-channel mean subtracted, blocks along the head dimension"), lambda: None
     if name == "refresh":
         from kohakuwullm_amd.models.mlp import MXFP8SwiGLU
         from kohakuwullm_amd.models.mxfp8_swap import refresh_mxfp8_weights
@@ -358,6 +375,7 @@ def build_workload(name: str, dev):
 STREAM_METRICS = {
     "norm": ("RMSNorm -> MXFP8 producer fwd+bwd GB/s", "f32 arithmetic on bf16, fp64 sum of squares"),
     "dispatch": ("expert dispatch (counts, sort, combine fwd+bwd) GB/s", "int32 indices, f32 arithmetic on bf16 rows"),
+    "heads": ("MXFP8 attention-operand quantizer GB/s", "bf16 - f32 mean -> e4m3 + ue8m0"),
     "refresh": ("MXFP8 weight requantization (row + column axis) GB/s", "bf16 -> e4m3 + ue8m0"),
 }
 
@@ -367,7 +385,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh"),
+    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh", "heads"),
                     help="ffn (default) is the configuration the headline metric is quoted on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")

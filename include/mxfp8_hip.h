@@ -91,6 +91,18 @@ int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t l
                      uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
 
 /*
+ * (T, H, D) attention operand -> e4m3 codes (T, H, D) and UE8M0 bytes (T, H, D/32), both
+ * contiguous, blocks of 32 along D (the contraction axis of QK^T).  x has unit stride along D,
+ * stride_h between heads and stride_t between tokens (elements): a slice of a fused projection
+ * output is quantized where it lies.  mu: optional (H, D) fp32 mean, subtracted in fp32 before
+ * the block maximum is taken (NULL: none).  D % 32 == 0.
+ * Replaces _quant_heads_kernel / quantize_heads
+ * (src/kohakuwullm/kernels/mxfp8/attention_quant.py:17-118).
+ */
+int mx_quantize_heads(const void *x, int x_dtype, int64_t T, int64_t H, int64_t D, int64_t stride_t, int64_t stride_h,
+                      const float *mu, uint8_t *q, uint8_t *s, void *stream);
+
+/*
  * mx_quantize_dual of `count` matrices behind one launch (one per 24 of them): the
  * once-per-optimizer-step requantization of every weight matrix of a model, which the
  * reference performs as one launch per matrix and axis from refresh_mxfp8_weights

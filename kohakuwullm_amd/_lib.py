@@ -30,6 +30,7 @@ SIGNATURES = {
     "mx_quantize_rows": (_ci, [_p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_quantize_cols": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
+    "mx_quantize_heads": (_ci, [_p, _ci, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p]),
     "mx_quantize_dual_batch": (_ci, [_p, _ci, _ci, _p]),
     "mx_swiglu_quantize_rows": (_ci, [_p, _p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_swiglu_quantize_dual": (_ci, [_p, _ci, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),

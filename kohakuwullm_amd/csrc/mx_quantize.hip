@@ -78,6 +78,62 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(const void *__restrict_
     }
 }
 
+// (T, H, D) attention operand, blocks along D: the row quantizer with a head stride and an
+// optional per-(head, channel) fp32 mean subtracted in registers (the smoothing of the MXFP8
+// QK^T operands: no shifted copy of the operand reaches memory).  Outputs are contiguous
+// (T, H*D) codes and (T, H*D/32) scale bytes.  D % 32 == 0, so a chunk of 8 stays inside a head.
+template <int DT, bool SMOOTH>
+__global__ __launch_bounds__(256) void quant_heads_kernel(const void *__restrict__ x, uint32_t chunks_per_row,
+                                                           uint32_t chunks_per_head, int64_t stride_t, int64_t stride_h,
+                                                           const float *__restrict__ mu, uint8_t *__restrict__ q,
+                                                           uint8_t *__restrict__ s, uint32_t total_chunks,
+                                                           int pack_scales) {
+    typedef typename Elem<DT>::type T;
+    constexpr int U = 4;
+    const int lane = threadIdx.x & 63;
+    const uint32_t base = blockIdx.x * (uint32_t)(U * 256) + threadIdx.x;
+    float v[U][8];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t chunk = base + u * 256;
+        ok[u] = chunk < total_chunks;
+        const uint32_t row = chunk / chunks_per_row, col = chunk - row * chunks_per_row;
+        const uint32_t head = col / chunks_per_head, d = col - head * chunks_per_head;
+        if (ok[u]) {
+            Elem<DT>::load8((const T *)x + (int64_t)row * stride_t + (int64_t)head * stride_h + (int64_t)d * 8, v[u]);
+            if (SMOOTH) {
+                const v4f a = ((const v4f *)(mu + (int64_t)col * 8))[0], b = ((const v4f *)(mu + (int64_t)col * 8))[1];
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[u][i] -= a[i], v[u][4 + i] -= b[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[u][i] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t chunk = base + u * 256;
+        float amax = quad_max(amax8(v[u]));
+        uint32_t byte = scale_byte(amax);
+        float inv = inv_scale(byte);
+        uint32_t packed = gather_row_scales(byte, lane);
+        if (ok[u]) {
+            v2i codes;
+            codes[0] = (int)pack4_e4m3(v[u][0] * inv, v[u][1] * inv, v[u][2] * inv, v[u][3] * inv);
+            codes[1] = (int)pack4_e4m3(v[u][4] * inv, v[u][5] * inv, v[u][6] * inv, v[u][7] * inv);
+            *(v2i *)(q + (int64_t)chunk * 8) = codes;
+            bool group_full = (chunk | 15u) < total_chunks;
+            if (pack_scales && group_full) {
+                if ((lane & 15) == 0) *(uint32_t *)(s + (chunk >> 2)) = packed;
+            } else if ((lane & 3) == 0) {
+                s[chunk >> 2] = (uint8_t)byte;
+            }
+        }
+    }
+}
+
 // Any strides: one thread per block.  The slow path for doubly-strided views.
 template <int DT>
 __global__ __launch_bounds__(256) void quant_rows_generic_kernel(const void *__restrict__ x, int64_t M, int64_t KB,
@@ -613,6 +669,38 @@ extern "C" int mx_quantize_rows(const void *x, int x_dtype, int64_t M, int64_t K
     case MX_FP16: return launch_rows<MX_FP16>(x, M, K, sx_row, sx_col, q, ldq, s, lds, st);
     case MX_FP32: return launch_rows<MX_FP32>(x, M, K, sx_row, sx_col, q, ldq, s, lds, st);
     default: return MX_EINVAL;
+    }
+}
+
+template <int DT>
+static int launch_heads(const void *x, int64_t T, int64_t H, int64_t D, int64_t stride_t, int64_t stride_h,
+                        const float *mu, uint8_t *q, uint8_t *s, hipStream_t st) {
+    const uint32_t cpr = (uint32_t)(H * D / 8), cph = (uint32_t)(D / 8), total = (uint32_t)(T * (H * D / 8));
+    const unsigned grid = (total + 4 * 256 - 1) / (4 * 256);
+    // the outputs are contiguous, so a 16-lane group's 4 scale bytes are one aligned dword whatever the row length
+    const int pack = aligned(s, 4);
+    if (mu)
+        quant_heads_kernel<DT, true><<<dim3(grid), dim3(256), 0, st>>>(x, cpr, cph, stride_t, stride_h, mu, q, s, total, pack);
+    else
+        quant_heads_kernel<DT, false><<<dim3(grid), dim3(256), 0, st>>>(x, cpr, cph, stride_t, stride_h, mu, q, s, total, pack);
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+extern "C" int mx_quantize_heads(const void *x, int x_dtype, int64_t T, int64_t H, int64_t D, int64_t stride_t,
+                                 int64_t stride_h, const float *mu, uint8_t *q, uint8_t *s, void *stream) {
+    if (T < 0 || H < 0 || D < 0 || D % MX_BLOCK || (H > 1 && stride_h < D) || stride_t < 0) return MX_EINVAL;
+    if (x_dtype != MX_BF16 && x_dtype != MX_FP16 && x_dtype != MX_FP32) return MX_EINVAL;
+    if (T == 0 || H == 0 || D == 0) return MX_OK;
+    if (!x || !q || !s) return MX_EINVAL;
+    if (!aligned(x, 16) || (stride_t * esize(x_dtype)) % 16 || (stride_h * esize(x_dtype)) % 16 || !aligned(q, 8) ||
+        (mu && !aligned(mu, 16)) || T * (H * D / 8) >= (int64_t)0x7FFFFF00)
+        return MX_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    switch (x_dtype) {
+    case MX_BF16: return launch_heads<MX_BF16>(x, T, H, D, stride_t, stride_h, mu, q, s, st);
+    case MX_FP16: return launch_heads<MX_FP16>(x, T, H, D, stride_t, stride_h, mu, q, s, st);
+    default: return launch_heads<MX_FP32>(x, T, H, D, stride_t, stride_h, mu, q, s, st);
     }
 }
 

@@ -16,6 +16,7 @@ Reference lines followed (paths relative to the reference tree):
   ``src/kohakuwullm/kernels/mxfp8/moe.py:408-433``
 * error metrics ........... ``src/kohakuwullm/bench/core/timing.py:201-228``
 * expert sort (CPU) ....... ``src/kohakuwullm/kernels/moe/moe_dispatch.py:264-282``
+* attention operand ....... ``src/kohakuwullm/kernels/mxfp8/attention_quant.py:17-118``
 * expert counts, combine .. ``src/kohakuwullm/models/components/moe.py:38-46``,
   ``src/kohakuwullm/kernels/moe/moe_dispatch.py:60-131,203-220``
 * RMSNorm -> MXFP8 ........ ``src/kohakuwullm/kernels/elementwise/rmsnorm.py:20-128``,
@@ -142,6 +143,17 @@ def swiglu_quantize_rows(gate: torch.Tensor, up: torch.Tensor) -> tuple[torch.Te
     )
     assert rc == 0
     return q, s
+
+
+def quantize_heads(x: torch.Tensor, mu: torch.Tensor | None = None):
+    """``(T, H, D)`` -> codes ``(T, H, D)`` uint8, scales ``(T, H, D // 32)``; blocks along D (attention_quant.py:17-118).
+
+    ``mu`` ``(H, D)`` fp32 is subtracted in fp32 before the block maximum is taken.
+    """
+    t, h, d = x.shape
+    y = x.float() if mu is None else x.float() - mu.float()[None]
+    q, s = quantize_rows(y.reshape(t, h * d).contiguous())
+    return q.view(t, h, d), s.view(t, h, d // BLOCK_SCALE)
 
 
 def quantize_rows_torch(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

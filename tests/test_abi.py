@@ -87,3 +87,7 @@ def test_entry_points_validate_before_launch():
     assert lib.mx_quantize_dual_batch(ctypes.byref(probs), 1, 7, None) == _lib.MX_EINVAL  # dtype
     probs[1] = _lib.QuantProblem(None, None, None, None, None, 64, 64, 64, 64, 2, 64, 2)  # null operands
     assert lib.mx_quantize_dual_batch(ctypes.byref(probs), 2, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_quantize_heads(None, 0, 8, 4, 48, 192, 48, None, None, None, None) == _lib.MX_EINVAL  # D % 32
+    assert lib.mx_quantize_heads(None, 0, 8, 4, 64, 256, 32, None, None, None, None) == _lib.MX_EINVAL  # heads overlap
+    assert lib.mx_quantize_heads(None, 0, 0, 4, 64, 256, 64, None, None, None, None) == _lib.MX_OK
+    assert lib.mx_quantize_heads(None, 0, 8, 4, 64, 256, 64, None, None, None, None) == _lib.MX_EINVAL  # null operands

@@ -189,3 +189,59 @@ def test_full_size_properties(oracle):
     # block amax lands in the top binade of its scale
     deq = q.float().reshape(16384, -1, 32).abs().amax(-1)
     assert (deq <= 448).all() and (deq >= 224).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("t,h,d", [(1, 1, 32), (77, 3, 64), (500, 16, 128), (33, 5, 96), (4096, 4, 128)])
+def test_quantize_heads_matches_oracle(oracle, dtype, t, h, d):
+    from kohakuwullm_amd.kernels.mxfp8.attention_quant import column_mean, quantize_heads
+
+    g = torch.Generator().manual_seed(SEED)
+    x = (torch.randn(t, h, d, generator=g) * 3.0 + 0.5).to(dtype)
+    if t > 2:
+        x[1] = 0.0
+    mu = torch.randn(h, d, generator=g)
+    for shift in (None, mu):
+        q, s = quantize_heads(x.to(DEV), None if shift is None else shift.to(DEV))
+        ref_q, ref_s = oracle.quantize_heads(x, shift)
+        assert q.shape == (t, h, d) and s.shape == (t, h, d // 32) and q.dtype == torch.float8_e4m3fn
+        assert torch.equal(q.view(torch.uint8).cpu(), ref_q) and torch.equal(s.cpu(), ref_s)
+    assert torch.allclose(column_mean(x.to(DEV)).cpu(), x.float().mean(0), atol=1e-5) and column_mean(x.to(DEV)).dtype == torch.float32
+
+
+def test_quantize_heads_reads_projection_slices_in_place_and_checks_input(oracle):
+    """q / k of a fused (T, (Hq + 2 Hkv) D) projection output, quantized where they lie; odd layouts are copied."""
+    from kohakuwullm_amd import _lib
+    from kohakuwullm_amd.kernels.mxfp8.attention_quant import quantize_heads
+
+    g = torch.Generator().manual_seed(SEED)
+    t, hq, hkv, d = 300, 16, 4, 128
+    qkv = torch.randn(t, (hq + 2 * hkv) * d, generator=g).bfloat16()
+    dev = qkv.to(DEV)
+    parts = {"q": (0, hq), "k": (hq * d, hkv)}
+    for lo, heads in parts.values():
+        view = dev[:, lo : lo + heads * d].view(t, heads, d)
+        assert not view.is_contiguous()
+        _lib.TIMER = []
+        q, s = quantize_heads(view)
+        calls, _lib.TIMER = _lib.TIMER, None
+        assert [c[0] for c in calls] == ["mx_quantize_heads"]
+        ref_q, ref_s = oracle.quantize_heads(qkv[:, lo : lo + heads * d].reshape(t, heads, d))
+        assert torch.equal(q.view(torch.uint8).cpu(), ref_q) and torch.equal(s.cpu(), ref_s)
+    # (H, T, D) storage seen as (T, H, D): unit stride along D, heads far apart
+    xt = torch.randn(hkv, t, d, generator=g).bfloat16()
+    q, s = quantize_heads(xt.to(DEV).permute(1, 0, 2))
+    ref_q, ref_s = oracle.quantize_heads(xt.permute(1, 0, 2))
+    assert torch.equal(q.view(torch.uint8).cpu(), ref_q) and torch.equal(s.cpu(), ref_s)
+    # D not innermost: copied, same result
+    xd = torch.randn(t, d, hkv, generator=g).bfloat16()
+    q, s = quantize_heads(xd.to(DEV).permute(0, 2, 1))
+    ref_q, ref_s = oracle.quantize_heads(xd.permute(0, 2, 1).contiguous())
+    assert torch.equal(q.view(torch.uint8).cpu(), ref_q) and torch.equal(s.cpu(), ref_s)
+    assert quantize_heads(dev[:0].view(0, 24, d))[0].shape == (0, 24, d)
+    with pytest.raises(ValueError):
+        quantize_heads(dev[:, : 4 * 48].view(t, 4, 48))
+    with pytest.raises(ValueError):
+        quantize_heads(dev[:, : 4 * d].view(t, 4, d), torch.zeros(4, d, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(_lib.MXFP8LibraryError):
+        quantize_heads(qkv[:, : 4 * d].view(t, 4, d))

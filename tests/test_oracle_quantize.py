@@ -181,3 +181,31 @@ def test_swizzle_matches_permute_formula(oracle):
     tiles = padded.view(rt, 128, ct, 4).permute(0, 2, 1, 3)
     ref = tiles.reshape(-1, 4, 32, 4).transpose(1, 2).reshape(-1, 32, 16).flatten()
     assert torch.equal(got, ref)
+
+
+def test_quantize_heads_against_torch_statement_and_invariants(oracle):
+    """The attention-operand quantizer: blocks along D with an fp32 mean taken off first.  Pinned by
+    the reference's own pure-torch quantizer formula on the shifted operand, by what a zero, an
+    equal and an exactly representable shift must give, and by the flat row quantizer when mu is absent."""
+    g = torch.Generator().manual_seed(SEED)
+    t, h, d = 37, 3, 64
+    x = (torch.randn(t, h, d, generator=g) * 2.0).bfloat16()
+    mu = torch.randn(h, d, generator=g) * 0.5
+    q, s = oracle.quantize_heads(x, mu)
+    ref_q, ref_s = oracle.quantize_rows_torch((x.float() - mu[None]).reshape(t, h * d))
+    assert torch.equal(q.reshape(t, h * d), ref_q) and torch.equal(s.reshape(t, -1), ref_s)
+    q0, s0 = oracle.quantize_heads(x)
+    flat_q, flat_s = oracle.quantize_rows(x.reshape(t, h * d))
+    assert torch.equal(q0.reshape(t, -1), flat_q) and torch.equal(s0.reshape(t, -1), flat_s)
+    qz, sz = oracle.quantize_heads(x, torch.zeros(h, d))
+    assert torch.equal(qz, q0) and torch.equal(sz, s0)
+    # an operand equal to its mean: every block empty (code 0, byte 19)
+    same = mu.bfloat16().float()
+    qe, se = oracle.quantize_heads(same[None].expand(t, h, d).bfloat16(), same)
+    assert not qe.any() and (se == 19).all()
+    # small integers shifted by an integer are exact in bf16: shifting operand and mean alike changes nothing
+    xi = torch.randint(-8, 9, (t, h, d), generator=g).float()
+    mi = torch.randint(-4, 5, (h, d), generator=g).float()
+    a = oracle.quantize_heads(xi.bfloat16(), mi)
+    b = oracle.quantize_heads((xi + 16.0).bfloat16(), mi + 16.0)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
