@@ -122,4 +122,14 @@ __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, b2));
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(v, off, 64);
+        if (lane >= off) v += up;
+    }
+    return v;
+}
+
 }  // namespace mx

@@ -135,6 +135,70 @@ __device__ __forceinline__ float row16_sum(float a) {
     return a + __shfl_xor(a, 8, 64);
 }
 
+// Per-expert prefix tables in LDS, built once per workgroup by its first wave (coalesced reads
+// of `offsets`, wave scans), so that finding the expert of a tile is a binary search or an
+// indexed read instead of a walk over `offsets` with one dependent scalar load per expert:
+// with 250 empty experts in front of the busy ones that walk cost every workgroup ~100 us per
+// launch.  More experts than the tables hold fall back to the walk.
+#define MX_TABLE_MAX 1024
+struct ExpertTable {
+    int a[MX_TABLE_MAX + 1];
+    int b[MX_TABLE_MAX + 1];
+    int n;
+};
+
+// a[e] = row tiles (of `bm` rows) of experts before e, b[e] = 128-row tiles of the padded token
+// axis before e, for e in [0, E]; n = E.
+__device__ __forceinline__ void build_row_tile_table(ExpertTable &tb, const int32_t *__restrict__ offsets, int E, int bm) {
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        int carry_t = 0, carry_p = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int rows = e < E ? offsets[e + 1] - offsets[e] : 0;
+            const int tiles = (rows + bm - 1) / bm, pads = (rows + 127) / 128;
+            const int it = wave_incl_scan(tiles, lane), ip = wave_incl_scan(pads, lane);
+            if (e < E) {
+                tb.a[e] = carry_t + it - tiles;
+                tb.b[e] = carry_p + ip - pads;
+            }
+            carry_t += __shfl(it, 63, 64);
+            carry_p += __shfl(ip, 63, 64);
+        }
+        if (lane == 0) {
+            tb.a[E] = carry_t;
+            tb.b[E] = carry_p;
+            tb.n = E;
+        }
+    }
+    __syncthreads();
+}
+
+// a[j] = the j-th expert with rows, b[j] = 128-token K stages of the experts before it; n = how many.
+__device__ __forceinline__ void build_live_table(ExpertTable &tb, const int32_t *__restrict__ offsets, int E) {
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const uint64_t below = lane ? ~0ull >> (64 - lane) : 0ull;
+        int carry_l = 0, carry_p = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int rows = e < E ? offsets[e + 1] - offsets[e] : 0;
+            const int pads = (rows + 127) / 128;
+            const int ip = wave_incl_scan(pads, lane);
+            const uint64_t mask = __ballot(rows > 0);
+            if (rows > 0) {
+                const int rank = carry_l + __builtin_popcountll(mask & below);
+                tb.a[rank] = e;
+                tb.b[rank] = carry_p + ip - pads;
+            }
+            carry_l += __builtin_popcountll(mask);
+            carry_p += __shfl(ip, 63, 64);
+        }
+        if (lane == 0) tb.n = carry_l;
+    }
+    __syncthreads();
+}
+
 template <typename S, int MODE, int CDT>
 struct GroupedProblem {
     struct Tile {
@@ -156,11 +220,17 @@ struct GroupedProblem {
     static constexpr int N_PER_TILE = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
-    __device__ GroupedProblem(const GroupedArgs &a)
-        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0), scan_pad(0) {}
+    const ExpertTable *tb;  // row-tile prefix table in LDS, or nullptr (more experts than it holds)
+
+    __device__ GroupedProblem(const GroupedArgs &a, const ExpertTable *table)
+        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0), scan_pad(0), tb(table) {}
 
     __device__ __forceinline__ bool next(Tile &t) {
-        const int total = p.tiles_n * p.tbound;
+        // With the table the number of real row tiles is known: ids cover exactly those, so the
+        // contiguous id ranges of the XCDs hold equal shares of real work.  (Over the host's bound,
+        // rows / BM + E row tiles, the ranges of the last XCDs hold only ids past the end: with 64
+        // experts at the benchmark's routing one XCD of eight had nothing to do.)
+        const int total = p.tiles_n * (tb ? tb->a[p.E] : p.tbound);
         const int per_xcd = total >> 3;
         while (next_id < total) {
             int id = next_id;
@@ -170,6 +240,23 @@ struct GroupedProblem {
             if (id < (per_xcd << 3)) id = (id & 7) * per_xcd + (id >> 3);
             const int rt = id / p.tiles_n;
             const int tn = id - rt * p.tiles_n;
+            if (tb) {
+                int lo = 0, hi = p.E;  // a[lo] <= rt < a[hi]: the last expert that starts at or before rt owns it
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) >> 1;
+                    if (tb->a[mid] <= rt) lo = mid;
+                    else hi = mid;
+                }
+                const int first = tb->a[lo];
+                t.expert = lo;
+                t.row0 = p.offsets[lo] + (rt - first) * S::BM;
+                t.end = p.offsets[lo + 1];
+                t.ppos = tb->b[lo] * 128 + (rt - first) * S::BM;
+                t.n0 = tn * N_PER_TILE;
+                t.kt0 = 0;
+                t.kt1 = p.K >> 7;
+                return true;
+            }
             if (rt < scan_tiles) {  // ids are monotonic per workgroup except across the XCD remap edge
                 scan_e = 0;
                 scan_tiles = 0;
@@ -655,7 +742,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t *__restrict
 template <typename S, int MODE, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void grouped_kernel(GroupedArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    GroupedProblem<S, MODE, CDT> prob(args);
+    __shared__ ExpertTable table;
+    const bool tabled = args.E <= MX_TABLE_MAX;
+    if (tabled) build_row_tile_table(table, args.offsets, args.E, S::BM);
+    GroupedProblem<S, MODE, CDT> prob(args, tabled ? &table : nullptr);
     persistent_gemm<S, K512>(prob, smem);
 }
 
@@ -713,9 +803,13 @@ struct WgradArgs {
 // Number of K slices per tile: as many as fill the GPU about twice over, at most 8, and 1 when
 // the tiles of the non-empty experts already fill three quarters of it.  Also counts the
 // non-empty experts.
-__device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, int &live) {
-    live = 0;
-    for (int e = 0; e < p.E; e++) live += p.offsets[e + 1] > p.offsets[e] ? 1 : 0;
+__device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, int &live, const ExpertTable *tb) {
+    if (tb) {
+        live = tb->n;
+    } else {
+        live = 0;
+        for (int e = 0; e < p.E; e++) live += p.offsets[e + 1] > p.offsets[e] ? 1 : 0;
+    }
     const int tiles = live * p.tiles_m * p.tiles_n;
     if (!p.slots || tiles == 0 || tiles * 4 >= workgroups * 3) return 1;
     int s = 2 * workgroups / tiles;
@@ -744,10 +838,13 @@ struct WgradProblem {
     // (b % 8) * (G / 8) + b / 8: the workgroups of one XCD take consecutive units, i.e. the tiles
     // of one (expert, K slice), which read the same operand panels, share that XCD's L2 (measured:
     // the kernel's fabric reads equal the operand bytes).
-    __device__ WgradProblem(const WgradArgs &a) : p(a), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0) {
+    const ExpertTable *tb;  // the experts with rows, in LDS, or nullptr (more experts than it holds)
+
+    __device__ WgradProblem(const WgradArgs &a, const ExpertTable *table)
+        : p(a), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0), tb(table) {
         const int g = (int)gridDim.x, b = (int)blockIdx.x;
         next_unit = (g & 7) == 0 ? (b & 7) * (g >> 3) + (b >> 3) : b;
-        slices = wgrad_slices(p, g, live);
+        slices = wgrad_slices(p, g, live, tb);
     }
 
     __device__ __forceinline__ void zero_slot(int slot) const {
@@ -764,7 +861,10 @@ struct WgradProblem {
             const int j = unit / per_live, r = unit - j * per_live;
             const int slice = r / per_e, rem = r - slice * per_e;  // slice-major: neighbours share operand panels
             // advance to the j-th non-empty expert (units, hence j, only grow for one workgroup)
-            while (true) {
+            if (tb) {
+                scan_e = tb->a[j];
+                scan_tiles = tb->b[j];
+            } else while (true) {
                 const int rows = p.offsets[scan_e + 1] - p.offsets[scan_e];
                 if (rows > 0 && scan_live == j) break;
                 scan_tiles += (rows + 127) / 128;
@@ -875,50 +975,61 @@ __global__ __launch_bounds__(256) void wgrad_zero_kernel(WgradArgs p, int chunks
 template <typename S, int CDT>
 __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    WgradProblem<S, CDT> prob(args);
+    __shared__ ExpertTable table;
+    const bool tabled = args.E <= MX_TABLE_MAX;
+    if (tabled) build_live_table(table, args.offsets, args.E);
+    WgradProblem<S, CDT> prob(args, tabled ? &table : nullptr);
     persistent_gemm<S, SCALES_DWORD>(prob, smem);
 }
 
 // Adds the K slices of every tile of every non-empty expert, in slice order, and stores dW.
-// One block per (tile of a non-empty expert, i), numbered compactly as in the GEMM; the grid is
-// sized for E experts, so blocks past the non-empty ones, and all blocks when the GEMM kept its
-// tiles whole, have nothing to do.
+// One unit per (tile of a non-empty expert, i), numbered compactly as in the GEMM; the host does
+// not know how many experts have rows, so a fixed number of workgroups stride over the units
+// (none when the GEMM kept its tiles whole).
 template <typename S, int CDT>
 __global__ __launch_bounds__(S::NTHR) void wgrad_reduce_kernel(WgradArgs p, int workgroups) {
+    __shared__ ExpertTable table;
+    const bool tabled = p.E <= MX_TABLE_MAX;
+    if (tabled) build_live_table(table, p.offsets, p.E);
     int live;
-    const int slices = wgrad_slices(p, workgroups, live);
+    const int slices = wgrad_slices(p, workgroups, live, tabled ? &table : nullptr);
     if (slices == 1) return;
     const int per_e = p.tiles_m * p.tiles_n;
-    const int id = blockIdx.x / S::MT, i = blockIdx.x % S::MT;
-    const int j = id / per_e, rem = id - j * per_e;
-    if (j >= live) return;
-    int e = 0;
-    for (int seen = 0;; e++) {
-        if (p.offsets[e + 1] > p.offsets[e]) {
-            if (seen == j) break;
-            seen++;
-        }
-    }
     const int tid = threadIdx.x;
-    v4f sum[S::NT];
-#pragma unroll
-    for (int jj = 0; jj < S::NT; jj++) sum[jj] = v4f{0.f, 0.f, 0.f, 0.f};
-    for (int sl = 0; sl < slices; sl++) {
-        const v4f *src = (const v4f *)p.ws + (int64_t)((j * per_e + rem) * slices + sl) * (S::BM * S::BN / 4);
-#pragma unroll
-        for (int jj = 0; jj < S::NT; jj++) sum[jj] += src[(i * S::NT + jj) * S::NTHR + tid];
-    }
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / S::WGN, wn = wave % S::WGN;
-    const int n = (rem % p.tiles_n) * S::BN + wn * S::WTN + 8 * (lane & 15);
+    for (int unit = blockIdx.x; unit < live * per_e * S::MT; unit += gridDim.x) {
+        const int id = unit / S::MT, i = unit % S::MT;
+        const int j = id / per_e, rem = id - j * per_e;
+        int e = 0;
+        if (tabled) {
+            e = table.a[j];
+        } else {
+            for (int seen = 0;; e++) {
+                if (p.offsets[e + 1] > p.offsets[e]) {
+                    if (seen == j) break;
+                    seen++;
+                }
+            }
+        }
+        v4f sum[S::NT];
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-        const int m = (rem / p.tiles_n) * S::BM + wm * S::WTM + 16 * i + 4 * (lane >> 4) + v;
-        if (m < p.N && n < p.Kout) {
-            const v4f lo = {sum[0][v], sum[1][v], sum[2][v], sum[3][v]};
-            const v4f hi = {sum[4][v], sum[5][v], sum[6][v], sum[7][v]};
-            store8<CDT>(p.dw, (int64_t)e * p.stride_dwe + (int64_t)m * p.lddw + n, lo, hi, p.Kout - n < 8 ? p.Kout - n : 8,
-                        p.c_vec != 0);
+        for (int jj = 0; jj < S::NT; jj++) sum[jj] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int sl = 0; sl < slices; sl++) {
+            const v4f *src = (const v4f *)p.ws + (int64_t)((j * per_e + rem) * slices + sl) * (S::BM * S::BN / 4);
+#pragma unroll
+            for (int jj = 0; jj < S::NT; jj++) sum[jj] += src[(i * S::NT + jj) * S::NTHR + tid];
+        }
+        const int n = (rem % p.tiles_n) * S::BN + wn * S::WTN + 8 * (lane & 15);
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int m = (rem / p.tiles_n) * S::BM + wm * S::WTM + 16 * i + 4 * (lane >> 4) + v;
+            if (m < p.N && n < p.Kout) {
+                const v4f lo = {sum[0][v], sum[1][v], sum[2][v], sum[3][v]};
+                const v4f hi = {sum[4][v], sum[5][v], sum[6][v], sum[7][v]};
+                store8<CDT>(p.dw, (int64_t)e * p.stride_dwe + (int64_t)m * p.lddw + n, lo, hi, p.Kout - n < 8 ? p.Kout - n : 8,
+                            p.c_vec != 0);
+            }
         }
     }
 }
@@ -1126,7 +1237,9 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
     if ((int64_t)a.E * chunks >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
     wgrad_zero_kernel<CDT><<<dim3((unsigned)(a.E * chunks)), dim3(256), 0, st>>>(a, chunks);
     kern<<<grid, block, S::LDS_BYTES, st>>>(a);
-    if (a.slots) wgrad_reduce_kernel<S, CDT><<<dim3((unsigned)(work * S::MT)), block, 0, st>>>(a, (int)grid.x);
+    // tiles are only split while (tiles x slices) fit the 2 * cus slots, so 4 * cus workgroups cover every unit at once
+    const int64_t units = work * S::MT < 4 * (int64_t)cus ? work * S::MT : 4 * (int64_t)cus;
+    if (a.slots) wgrad_reduce_kernel<S, CDT><<<dim3((unsigned)units), block, 0, st>>>(a, (int)grid.x);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 

@@ -517,20 +517,32 @@ __global__ __launch_bounds__(256) void quant_cols_grouped_kernel(GroupedQuantArg
     __shared__ __attribute__((aligned(4))) uint8_t tscale[QC_TILE * 4];
     const int t = threadIdx.x;
     const int rt = blockIdx.y;
-    // tile_owner: experts whose tiles all precede rt
-    int e = 0, before = 0, start = 0, end = 0;
-    bool found = false;
-    for (; e < a.E; e++) {
-        start = a.offsets[e];
-        end = a.offsets[e + 1];
-        const int tiles = (end - start + QC_TILE - 1) / QC_TILE;
-        if (rt < before + tiles) {
-            found = true;
-            break;
+    // tile_owner: the expert whose tiles contain rt.  The first wave looks at 64 experts at a time
+    // (one coalesced read of `offsets`, a wave scan of their tile counts) instead of walking the
+    // experts with a dependent scalar load each: with hundreds of experts, most of them empty,
+    // that walk took longer than the tile itself.
+    __shared__ int owner[4];
+    if (t < 64) {
+        int carry = 0;
+        bool done = false;
+        for (int e0 = 0; e0 < a.E && !done; e0 += 64) {
+            const int e = e0 + t;
+            const int lo = e < a.E ? a.offsets[e] : 0, hi = e < a.E ? a.offsets[e + 1] : 0;
+            const int tiles = (hi - lo + QC_TILE - 1) / QC_TILE;
+            const int incl = wave_incl_scan(tiles, t);
+            const int first = carry + incl - tiles;
+            const bool mine = e < a.E && rt >= first && rt < first + tiles;
+            if (__ballot(mine)) {
+                if (mine) owner[0] = e, owner[1] = first, owner[2] = lo, owner[3] = hi;
+                done = true;
+            }
+            carry += __shfl(incl, 63, 64);
         }
-        before += tiles;
+        if (!done && t == 0) owner[0] = -1;
     }
-    if (!found) return;  // beyond the last real tile: that part of the padded space is never read
+    __syncthreads();
+    if (owner[0] < 0) return;  // beyond the last real tile: that part of the padded space is never read
+    const int before = owner[1], start = owner[2], end = owner[3];
     const int row_base = start + (rt - before) * QC_TILE;
     const int64_t k0 = (int64_t)blockIdx.x * QC_TILE;
     const int64_t col = k0 + (t & 15) * 8;

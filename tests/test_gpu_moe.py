@@ -46,6 +46,11 @@ COUNT_CASES = [
     [64, 64, 64, 64],
     [0, 0, 5, 0],
     [700],
+    # many experts, most of them empty, the busy ones behind long runs of empties: the owner of a
+    # tile is found through the per-workgroup expert tables (more than one 64-expert chunk)
+    [0] * 70 + [200] + [0] * 130 + [129, 1] + [0] * 50,
+    # more experts than the tables hold: the kernels fall back to walking `offsets`
+    [0] * 1040 + [90, 0, 33] + [0] * 20,
 ]
 
 
@@ -133,7 +138,7 @@ def _padded_cols_ref(oracle, rows_fp32, offsets, dtype=torch.bfloat16):
     return q, s, valid
 
 
-@pytest.mark.parametrize("counts", COUNT_CASES[:3])
+@pytest.mark.parametrize("counts", COUNT_CASES[:3] + COUNT_CASES[4:])
 def test_grouped_token_axis_quantizer_and_wgrad(oracle, counts):
     from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_wgrad, quantize_mx_cols_grouped
 
@@ -234,7 +239,8 @@ def _expert_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
     return dict(out=out, pre=pre, hq=hq, hs=hs, dx=dx, dgate=dgate, dw_in=dw_in, dw_out=dw_out)
 
 
-@pytest.mark.parametrize("counts,top_k", [([300, 0, 1, 257, 0, 130], 2), ([256, 256], 1)])
+@pytest.mark.parametrize("counts,top_k", [([300, 0, 1, 257, 0, 130], 2), ([256, 256], 1),
+                                          ([0] * 70 + [200] + [0] * 130 + [129, 1] + [0] * 50, 1)])
 @pytest.mark.parametrize("dout_scale", [1.0, 2.0**-20])
 def test_fused_experts_fwd_bwd(oracle, counts, top_k, dout_scale):
     from kohakuwullm_amd.kernels.mxfp8.moe import (
