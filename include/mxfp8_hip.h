@@ -85,6 +85,15 @@ int mx_quantize_cols(const void *x, int x_dtype, int64_t M, int64_t K, int64_t l
  * as mx_quantize_cols.  M % 32 == 0 and K % 32 == 0.
  * Replaces the pair of quantize calls an activation needs when it feeds both a
  * forward/dgrad GEMM (blocks along its K) and a wgrad GEMM (blocks along tokens).
+ *
+ * Stage-major codes.  A code matrix of R rows and C > 128 columns whose leading dimension is
+ * given as exactly 128 is stored as C/128 panels: panel p (columns 128 p .. 128 p + 127) at byte
+ * offset p * R * 128, row r of it at r * 128.  C % 128 == 0.  A K stage of a GEMM tile (256
+ * rows x 128 bytes) is then one contiguous run instead of 256 rows a pitch apart, which DRAM
+ * serves 3-4 % faster on long contractions.  Accepted for qT here and in
+ * mx_swiglu_quantize_dual, for q and qT in mx_swiglu_bwd_quantize_dual, and for the A and B
+ * codes of mx_gemm_nt / mx_gemm_nt_batch.  Scale bytes keep their row-major layout.  The
+ * layout has no counterpart in the reference; the public (rows, K) layouts are the default.
  */
 int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                      uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
@@ -196,7 +205,8 @@ int mx_unswizzle_scales(const uint8_t *swizzled, int64_t rows, int64_t cols, uin
  * even).  A: codes (M,K) pitch lda + scales (M,K/32) pitch ldas; B: codes (N,K)
  * pitch ldb + scales (N,K/32) pitch ldbs; both K-minor.  K % 32 == 0.
  * One entry serves forward (X W^T), dgrad (dY (W^T)^T) and wgrad (dY^T (X^T)^T)
- * because the quantizers deliver every operand K-minor.
+ * because the quantizers deliver every operand K-minor.  lda == 128 (ldb == 128) with
+ * K > 128 reads A (B) in the stage-major layout described at mx_quantize_dual (K % 128 == 0).
  * Replaces mxfp8_matmul_pq / _mxfp8_matmul_pq
  * (src/kohakuwullm/kernels/mxfp8/quantize.py:242-371) and the cuBLAS route
  * mxfp8_mm_swizzled (src/kohakuwullm/kernels/mxfp8/interop.py:51-122).

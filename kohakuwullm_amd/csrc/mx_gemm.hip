@@ -33,6 +33,10 @@ struct DenseArgs {
     int dp_tiles, sk_tiles, sk_q;
     float *sk_ws;
     int xcds;  // XCDs this problem's workgroups are spread over (8; fewer inside a batched launch)
+    // Stage-major operands (0: row-major).  a_ks: A is stored as K/128 panels of 128 bytes of every
+    // row, panel kt at kt * a_ks, row m of it at m * 128 (lda is 128 then); b_ks likewise.  A K stage
+    // of a tile is then one contiguous run instead of 256 rows a pitch apart.
+    int64_t a_ks, b_ks;
 };
 
 // Whether tile_of staggers the column walk (see there): up to 64 K stages per tile.
@@ -101,6 +105,8 @@ struct DenseProblem {
         const Lane L = opaque(L0);
         c.a_base = p.aq + (int64_t)t.m0 * p.lda;
         c.b_base = p.bq + (int64_t)t.n0 * p.ldb;
+        c.a_ks = p.a_ks ? p.a_ks : 128;
+        c.b_ks = p.b_ks ? p.b_ks : 128;
         c.kt0 = t.kt0;
         c.kt1 = t.kt1;
         c.tail_bytes = p.K & 127;
@@ -461,7 +467,7 @@ template <int CDT>
 static int gemm_dispatch(DenseArgs a, hipStream_t st) {
     const int64_t M = a.M, N = a.N;
     if (!tiled_ok(a)) {
-        if (a.accumulate) return MX_EUNSUPPORTED;
+        if (a.accumulate || a.a_ks || a.b_ks) return MX_EUNSUPPORTED;  // the element-wise kernel reads row-major only
         int64_t blocks = (M * N + 255) / 256;
         if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
         gemm_nt_generic_kernel<CDT><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a.aq, a.as, a.bq, a.bs, a.c, M, N, a.K,
@@ -606,8 +612,11 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
 
 static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs, void *c,
                      int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldas, int64_t ldb, int64_t ldbs, int64_t ldc) {
-    if (M < 0 || N < 0 || K < 0 || K % MX_BLOCK || lda < K || ldb < K || ldas < K / MX_BLOCK || ldbs < K / MX_BLOCK ||
-        ldc < N || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
+    // a leading dimension of exactly 128 with K > 128 is the stage-major layout (see the header)
+    const bool a_panels = lda == 128 && K > 128, b_panels = ldb == 128 && K > 128;
+    if (M < 0 || N < 0 || K < 0 || K % MX_BLOCK || (lda < K && !a_panels) || (ldb < K && !b_panels) ||
+        ((a_panels || b_panels) && K % 128) || ldas < K / MX_BLOCK || ldbs < K / MX_BLOCK || ldc < N ||
+        M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
         return MX_EINVAL;
     a.aq = aq, a.as = as, a.bq = bq, a.bs = bs, a.c = c;
     a.M = (int)M, a.N = (int)N, a.K = (int)K;
@@ -618,6 +627,8 @@ static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const u
     a.dp_tiles = a.sk_tiles = a.sk_q = 0;
     a.sk_ws = nullptr;
     a.xcds = 8;
+    a.a_ks = a_panels ? M * 128 : 0;
+    a.b_ks = b_panels ? N * 128 : 0;
     return MX_OK;
 }
 

@@ -134,6 +134,7 @@ __device__ __forceinline__ int b_row_of_lds(int r) {
 template <typename S>
 struct IssueCtx {
     const uint8_t *a_base, *b_base;
+    int64_t a_ks = 128, b_ks = 128;  // bytes from one K stage of an operand to the next (128: row-major)
     uint32_t a_voff[S::QA], b_voff[S::QB];
     const uint8_t *srow0, *srow1;  // scale rows tid and tid + NTHR of the [A rows; B rows] list
     int kt0, kt1;                  // K range in 128-byte stages (absolute)
@@ -171,8 +172,8 @@ __device__ __forceinline__ void issue_stage(const IssueCtx<S> &c, const Lane &L,
                                             int buf) {
     // The stage's base address is forced into SGPRs so each load is "scalar base + 32-bit
     // lane offset" and costs no 64-bit vector address arithmetic.
-    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt * 128);
-    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt * 128);
+    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt * c.a_ks);
+    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt * c.b_ks);
     const uint32_t la = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf * S::DATA_A + L.wave * 1024);
     const uint32_t lb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf * S::DATA_B + L.wave * 1024);
 #pragma unroll
@@ -238,8 +239,8 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
                                               const int (&sb)[S::NT], v4f (&acc)[S::MT][S::NT],
                                               const IssueCtx<S> &c, const Lane &L, int kt_next, uint8_t *ldsA,
                                               uint8_t *ldsB, int buf_next) {
-    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt_next * 128);
-    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt_next * 128);
+    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt_next * c.a_ks);
+    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt_next * c.b_ks);
     const uint32_t wa = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf_next * S::DATA_A + L.wave * 1024);
     const uint32_t wb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf_next * S::DATA_B + L.wave * 1024);
     constexpr int NQ = S::QA + S::QB;                      // copies this wave issues per stage

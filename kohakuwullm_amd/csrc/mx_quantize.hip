@@ -187,6 +187,10 @@ struct QuantTileOut {
     uint8_t *s;  // (M,K/32)
     int64_t lds;
     int pack_row_scales, pack_col_scales;
+    // Stage-major code layouts (0: row-major with the pitches above).  q_ks: 128-column panels
+    // of q, panel p at p * q_ks, row m of it at m * 128.  qT_ks: the same for qT (panels of 128
+    // of its M columns).  A GEMM then finds a K stage of a tile in one contiguous run.
+    int64_t q_ks, qT_ks;
 };
 
 // Quantizes the 128 x 128 tile held as v[8][8] per thread (rows m0 + rg*8 + i, columns
@@ -216,7 +220,7 @@ __device__ __forceinline__ void quant_tile(float (&v)[8][8], const QuantTileOut 
                 v2i codes;
                 codes[0] = (int)pack4_e4m3(v[i][0] * inv, v[i][1] * inv, v[i][2] * inv, v[i][3] * inv);
                 codes[1] = (int)pack4_e4m3(v[i][4] * inv, v[i][5] * inv, v[i][6] * inv, v[i][7] * inv);
-                *(v2i *)(o.q + (row0 + i) * o.ldq + col) = codes;
+                *(v2i *)(o.q + (o.q_ks ? (col >> 7) * o.q_ks + (row0 + i) * 128 + (col & 127) : (row0 + i) * o.ldq + col)) = codes;
                 uint8_t *sp = o.s + (row0 + i) * o.lds + (col >> 5);
                 bool full = kc0 + QC_TILE <= K;
                 if (o.pack_row_scales && full) {
@@ -265,7 +269,7 @@ __device__ __forceinline__ void quant_tile(float (&v)[8][8], const QuantTileOut 
             w[1] = a[1];
             w[2] = b[0];
             w[3] = b[1];
-            *(v4i *)(o.qT + (kc0 + kr) * o.ldqT + m0 + ch * 16) = w;
+            *(v4i *)(o.qT + (o.qT_ks ? (m0 >> 7) * o.qT_ks + (kc0 + kr) * 128 : (kc0 + kr) * o.ldqT + m0) + ch * 16) = w;
         }
     }
     if (t < QC_TILE && kc0 + t < K) {
@@ -419,9 +423,9 @@ __global__ __launch_bounds__(256) void swiglu_bwd_quant_dual_kernel(const void *
     // Columns at or beyond H inside the gate-half tile are masked by passing K = H.
     quant_tile<true>(v, o, M, H, m0, k0, tile, tscale);
     QuantTileOut o2 = o;
-    o2.q += H;
+    o2.q += o.q_ks ? (H >> 7) * o.q_ks : H;
     o2.s += H / MX_BLOCK;
-    o2.qT += H * o.ldqT;
+    o2.qT += o.qT_ks ? H * 128 : H * o.ldqT;
     o2.sT += H * o.ldsT;
     quant_tile<true>(w, o2, M, H, m0, k0, tile, tscale);
 }
@@ -622,10 +626,15 @@ static int launch_rows(const void *x, int64_t M, int64_t K, int64_t sx_row, int6
     return MX_OK;
 }
 
+// A leading dimension of exactly 128 for a matrix wider than 128 columns asks for the stage-major
+// layout: 128-column panels, each holding every row (pitch 128), panel p at p * rows * 128.
+static bool stage_major(int64_t ld, int64_t cols) { return ld == 128 && cols > 128; }
+
 static QuantTileOut tile_out(uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s,
-                             int64_t lds) {
+                             int64_t lds, int64_t q_ks = 0, int64_t qT_ks = 0) {
     QuantTileOut o;
     o.qT = qT, o.ldqT = ldqT, o.sT = sT, o.ldsT = ldsT, o.q = q, o.ldq = ldq, o.s = s, o.lds = lds;
+    o.q_ks = q_ks, o.qT_ks = qT_ks;
     o.pack_row_scales = s != nullptr && aligned(s, 4) && lds % 4 == 0;
     o.pack_col_scales = aligned(sT, 4) && ldsT % 4 == 0;
     return o;
@@ -633,10 +642,10 @@ static QuantTileOut tile_out(uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t lds
 
 template <int DT, bool DUAL>
 static int launch_cols(const void *x, int64_t M, int64_t K, int64_t ldx, uint8_t *qT, int64_t ldqT, uint8_t *sT,
-                       int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, hipStream_t st) {
+                       int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, hipStream_t st, int64_t qT_ks = 0) {
     dim3 grid((unsigned)((K + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
     if (grid.y > 65535u) return MX_EUNSUPPORTED;
-    quant_cols_kernel<DT, DUAL><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds));
+    quant_cols_kernel<DT, DUAL><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, 0, qT_ks));
     MX_LAUNCH_CHECK();
     return MX_OK;
 }
@@ -719,20 +728,23 @@ extern "C" int mx_quantize_heads(const void *x, int x_dtype, int64_t T, int64_t 
 extern "C" int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, uint8_t *q, int64_t ldq,
                                 uint8_t *s, int64_t lds, uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT,
                                 void *stream) {
-    if (M < 0 || K < 0 || M % MX_BLOCK || K % MX_BLOCK || ldx < K || ldq < K || lds < K / MX_BLOCK || ldqT < M ||
-        ldsT < M / MX_BLOCK)
+    const bool panels = stage_major(ldqT, M);  // qT as 128-token panels
+    if (M < 0 || K < 0 || M % MX_BLOCK || K % MX_BLOCK || ldx < K || ldq < K || lds < K / MX_BLOCK ||
+        (ldqT < M && !panels) || (panels && M % 128) || ldsT < M / MX_BLOCK)
         return MX_EINVAL;
     if (M == 0 || K == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
     if (!cols_vec_ok(x, x_dtype, K, ldx, qT, ldqT) || !aligned(q, 8) || ldq % 8) {
+        if (panels) return MX_EUNSUPPORTED;
         int rc = mx_quantize_rows(x, x_dtype, M, K, ldx, 1, q, ldq, s, lds, stream);
         if (rc != MX_OK) return rc;
         return mx_quantize_cols(x, x_dtype, M, K, ldx, qT, ldqT, sT, ldsT, stream);
     }
+    const int64_t ks = panels ? K * 128 : 0;
     switch (x_dtype) {
-    case MX_BF16: return launch_cols<MX_BF16, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
-    case MX_FP16: return launch_cols<MX_FP16, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
-    case MX_FP32: return launch_cols<MX_FP32, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st);
+    case MX_BF16: return launch_cols<MX_BF16, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st, ks);
+    case MX_FP16: return launch_cols<MX_FP16, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st, ks);
+    case MX_FP32: return launch_cols<MX_FP32, true>(x, M, K, ldx, qT, ldqT, sT, ldsT, q, ldq, s, lds, st, ks);
     default: return MX_EINVAL;
     }
 }
@@ -818,8 +830,9 @@ extern "C" int mx_swiglu_quantize_rows(const void *gate, const void *up, int dty
 extern "C" int mx_swiglu_quantize_dual(const void *gu, int dtype, int64_t M, int64_t H, int64_t ldgu, uint8_t *q,
                                        int64_t ldq, uint8_t *s, int64_t lds, uint8_t *qT, int64_t ldqT, uint8_t *sT,
                                        int64_t ldsT, void *stream) {
-    if (M < 0 || H < 0 || M % MX_BLOCK || H % MX_BLOCK || ldgu < 2 * H || ldq < H || lds < H / MX_BLOCK || ldqT < M ||
-        ldsT < M / MX_BLOCK)
+    const bool panels = stage_major(ldqT, M);  // qT as 128-token panels
+    if (M < 0 || H < 0 || M % MX_BLOCK || H % MX_BLOCK || ldgu < 2 * H || ldq < H || lds < H / MX_BLOCK ||
+        (ldqT < M && !panels) || (panels && M % 128) || ldsT < M / MX_BLOCK)
         return MX_EINVAL;
     if (M == 0 || H == 0) return MX_OK;
     if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
@@ -828,7 +841,7 @@ extern "C" int mx_swiglu_quantize_dual(const void *gu, int dtype, int64_t M, int
     dim3 grid((unsigned)((H + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
     if (grid.y > 65535u) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
-    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds);
+    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, 0, panels ? H * 128 : 0);
     if (dtype == MX_BF16) swiglu_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(gu, M, H, ldgu, o);
     else swiglu_quant_dual_kernel<MX_FP16><<<grid, dim3(256), 0, st>>>(gu, M, H, ldgu, o);
     MX_LAUNCH_CHECK();
@@ -838,8 +851,10 @@ extern "C" int mx_swiglu_quantize_dual(const void *gu, int dtype, int64_t M, int
 extern "C" int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, int64_t ldgu, int dtype,
                                            int64_t M, int64_t H, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
                                            uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream) {
-    if (M < 0 || H < 0 || M % MX_BLOCK || H % MX_BLOCK || lddh < H || ldgu < 2 * H || ldq < 2 * H ||
-        lds < 2 * H / MX_BLOCK || ldqT < M || ldsT < M / MX_BLOCK)
+    const bool q_panels = stage_major(ldq, 2 * H), qt_panels = stage_major(ldqT, M);
+    if (M < 0 || H < 0 || M % MX_BLOCK || H % MX_BLOCK || lddh < H || ldgu < 2 * H || (ldq < 2 * H && !q_panels) ||
+        (q_panels && H % 128) || lds < 2 * H / MX_BLOCK || (ldqT < M && !qt_panels) || (qt_panels && M % 128) ||
+        ldsT < M / MX_BLOCK)
         return MX_EINVAL;
     if (M == 0 || H == 0) return MX_OK;
     if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
@@ -849,7 +864,7 @@ extern "C" int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const v
     dim3 grid((unsigned)((H + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
     if (grid.y > 65535u) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
-    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds);
+    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, q_panels ? M * 128 : 0, qt_panels ? 2 * H * 128 : 0);
     if (H % 128) o.pack_row_scales = 0;  // the up half's scale columns start at H/32: keep dword stores aligned
     if (dtype == MX_BF16) swiglu_bwd_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);
     else swiglu_bwd_quant_dual_kernel<MX_FP16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);

@@ -21,48 +21,62 @@ from kohakuwullm_amd import _lib
 from kohakuwullm_amd.kernels.mxfp8.linear import compute_dtype
 from kohakuwullm_amd.kernels.mxfp8.quantize import (
     BLOCK_SCALE,
+    PANEL,
     mxfp8_matmul_pq,
     mxfp8_matmul_pq_batch,
     quantize_mx_dual,
+    stage_major_ok,
 )
 
 _FP8 = torch.float8_e4m3fn
 
 
-def swiglu_mx_dual(gu: torch.Tensor):
-    """``h = silu(gu[:, :H]) * gu[:, H:]`` as ``(q, s, qT, sT)``: blocks along H and along tokens."""
+def swiglu_mx_dual(gu: torch.Tensor, stage_major_t: bool = False):
+    """``h = silu(gu[:, :H]) * gu[:, H:]`` as ``(q, s, qT, sT)``: blocks along H and along tokens.
+
+    ``stage_major_t``: ``qT`` as ``(tokens // 128, H, 128)`` (see :func:`quantize_mx_dual`).
+    """
     m, two_h = gu.shape
     h = two_h // 2
     if two_h % 2 or h % BLOCK_SCALE or m % BLOCK_SCALE:
         raise ValueError(f"gu {tuple(gu.shape)}: tokens and hidden must be multiples of {BLOCK_SCALE}")
+    if stage_major_t and not stage_major_ok(m):
+        raise ValueError(f"stage_major_t needs the token count {m} to be a positive multiple of {PANEL}")
     _lib.require_gpu(gu, "gu")
     q = torch.empty(m, h, device=gu.device, dtype=_FP8)
     s = torch.empty(m, h // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
-    qt = torch.empty(h, m, device=gu.device, dtype=_FP8)
+    qt = torch.empty((m // PANEL, h, PANEL) if stage_major_t else (h, m), device=gu.device, dtype=_FP8)
     st = torch.empty(h, m // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
     _lib.invoke(
         "mx_swiglu_quantize_dual", m * h * (2 * gu.element_size() + 2 * (1 + 1 / BLOCK_SCALE)), gu,
         gu.data_ptr(), _lib.MX_DTYPE[gu.dtype], m, h, gu.stride(0), q.data_ptr(), h, s.data_ptr(), h // BLOCK_SCALE,
-        qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE,
+        qt.data_ptr(), PANEL if stage_major_t else m, st.data_ptr(), m // BLOCK_SCALE,
     )
     return q, s, qt, st
 
 
-def swiglu_bwd_mx_dual(dh: torch.Tensor, gu: torch.Tensor):
-    """SwiGLU backward emitted straight in MXFP8: ``dpre = [dgate | dup]`` as ``(q, s, qT, sT)``."""
+def swiglu_bwd_mx_dual(dh: torch.Tensor, gu: torch.Tensor, stage_major: bool = False):
+    """SwiGLU backward emitted straight in MXFP8: ``dpre = [dgate | dup]`` as ``(q, s, qT, sT)``.
+
+    ``stage_major``: ``q`` as ``(2H // 128, tokens, 128)`` and ``qT`` as ``(tokens // 128, 2H, 128)``
+    (tokens and H multiples of 128; see :func:`quantize_mx_dual`).
+    """
     m, two_h = gu.shape
     h = two_h // 2
     if dh.shape != (m, h) or h % BLOCK_SCALE or m % BLOCK_SCALE:
         raise ValueError(f"dh {tuple(dh.shape)} does not match gu {tuple(gu.shape)}")
+    if stage_major and not (stage_major_ok(m) and stage_major_ok(h)):
+        raise ValueError(f"stage_major needs tokens={m} and H={h} to be positive multiples of {PANEL}")
     _lib.require_gpu(gu, "gu")
-    q = torch.empty(m, two_h, device=gu.device, dtype=_FP8)
+    q = torch.empty((two_h // PANEL, m, PANEL) if stage_major else (m, two_h), device=gu.device, dtype=_FP8)
     s = torch.empty(m, two_h // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
-    qt = torch.empty(two_h, m, device=gu.device, dtype=_FP8)
+    qt = torch.empty((m // PANEL, two_h, PANEL) if stage_major else (two_h, m), device=gu.device, dtype=_FP8)
     st = torch.empty(two_h, m // BLOCK_SCALE, device=gu.device, dtype=torch.uint8)
     _lib.invoke(
         "mx_swiglu_bwd_quantize_dual", m * h * (3 * gu.element_size() + 4 * (1 + 1 / BLOCK_SCALE)), gu,
         dh.data_ptr(), dh.stride(0), gu.data_ptr(), gu.stride(0), _lib.MX_DTYPE[gu.dtype], m, h,
-        q.data_ptr(), two_h, s.data_ptr(), two_h // BLOCK_SCALE, qt.data_ptr(), m, st.data_ptr(), m // BLOCK_SCALE,
+        q.data_ptr(), PANEL if stage_major else two_h, s.data_ptr(), two_h // BLOCK_SCALE,
+        qt.data_ptr(), PANEL if stage_major else m, st.data_ptr(), m // BLOCK_SCALE,
     )
     return q, s, qt, st
 
@@ -109,17 +123,21 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         x2d = x.reshape(-1, shape[-1]).to(compute)
         if x2d.stride(-1) != 1:
             x2d = x2d.contiguous()
-        xq, xs, xtq, xts = quantize_mx_dual(x2d)
+        # The operands of the three backward products that go down in one launch (contractions of
+        # 8192 and 16384) are written stage-major: each K stage of a tile is then one contiguous run.
+        sm = x.dtype == compute and stage_major_ok(x2d.shape[0]) and stage_major_ok(w_out.shape[1])
+        xq, xs, xtq, xts = quantize_mx_dual(x2d, stage_major_t=sm)
         # GEMM, then one bandwidth-bound pass for SwiGLU and both casts: measured faster at the
         # benchmark shape (220 + 89 us) than the same work in the GEMM's epilogue
         # (fused_swiglu_projection: 329 us), whose vector ALU work cannot overlap the MFMAs.
         gu = mxfp8_matmul_pq(xq, xs, *in_f, compute)
-        hq, hs, htq, hts = swiglu_mx_dual(gu)
+        hq, hs, htq, hts = swiglu_mx_dual(gu, stage_major_t=sm)
         y = mxfp8_matmul_pq(hq, hs, *out_f, compute)
         if any(ctx.needs_input_grad):
             ctx.save_for_backward(xtq, xts, gu, htq, hts, *in_d, *out_d)
             ctx.compute = compute
             ctx.x_dtype = x.dtype
+            ctx.stage_major = sm
         return y.reshape(*shape[:-1], y.shape[-1])
 
     @staticmethod
@@ -127,9 +145,9 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         xtq, xts, gu, htq, hts, win_dq, win_ds, wout_dq, wout_ds = ctx.saved_tensors
         shape = dout.shape
         d2d = dout.reshape(-1, shape[-1]).to(ctx.compute).contiguous()
-        dq, ds, dtq, dts = quantize_mx_dual(d2d)
+        dq, ds, dtq, dts = quantize_mx_dual(d2d, stage_major_t=ctx.stage_major)
         dh = mxfp8_matmul_pq(dq, ds, wout_dq, wout_ds, ctx.compute)
-        pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu)
+        pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu, stage_major=ctx.stage_major)
         # The last three products are independent and none fills the GPU alone (dW has few
         # tiles with a long K): they go down together and share the GPU by work.
         wanted = [

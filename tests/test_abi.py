@@ -91,3 +91,9 @@ def test_entry_points_validate_before_launch():
     assert lib.mx_quantize_heads(None, 0, 8, 4, 64, 256, 32, None, None, None, None) == _lib.MX_EINVAL  # heads overlap
     assert lib.mx_quantize_heads(None, 0, 0, 4, 64, 256, 64, None, None, None, None) == _lib.MX_OK
     assert lib.mx_quantize_heads(None, 0, 8, 4, 64, 256, 64, None, None, None, None) == _lib.MX_EINVAL  # null operands
+    # a leading dimension of exactly 128 on a wider code matrix selects the stage-major layout: K % 128 then
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 256, 128, 8, 256, 8, 4, 0, None) == _lib.MX_OK  # A panels, empty
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 160, 128, 5, 160, 5, 4, 0, None) == _lib.MX_EINVAL  # K % 128
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 256, 64, 8, 256, 8, 4, 0, None) == _lib.MX_EINVAL  # lda < K, not 128
+    assert lib.mx_quantize_dual(None, 0, 0, 64, 64, None, 64, None, 2, None, 128, None, 0, None) == _lib.MX_OK
+    assert lib.mx_quantize_dual(None, 0, 160, 64, 64, None, 64, None, 2, None, 128, None, 5, None) == _lib.MX_EINVAL  # panels need M % 128
