@@ -26,6 +26,7 @@ from kohakuwullm_amd.kernels.mxfp8.quantize import (
     quantize_mx,
     quantize_mx_cols,
     quantize_mx_dual,
+    stage_major_ok,
 )
 
 # Alignment of FPROP's contraction axis (kept at the reference's value so `swap_mxfp8`
@@ -66,9 +67,12 @@ class _MXFP8Linear(torch.autograd.Function):
             x2d = x2d.contiguous()
         need_dw = ctx.needs_input_grad[1]
         fp8_wgrad = need_dw and x2d.shape[0] % BLOCK_SCALE == 0 and x2d.shape[0] > 0
+        # WGRAD contracts over the tokens (tens of thousands): its operands are written stage-major, a
+        # K stage of a tile in one contiguous run, when tokens come in whole panels and dout needs no padding
+        stage_major = fp8_wgrad and stage_major_ok(x2d.shape[0]) and pad_k.width == 0
         if fp8_wgrad:
             # One pass over x gives FPROP's operand and WGRAD's (blocks along tokens).
-            xq, xs, xtq, xts = quantize_mx_dual(x2d)
+            xq, xs, xtq, xts = quantize_mx_dual(x2d, stage_major_t=stage_major)
             saved_x = (xtq, xts)
         else:
             xq, xs = quantize_mx(x2d)
@@ -76,6 +80,7 @@ class _MXFP8Linear(torch.autograd.Function):
         out = mxfp8_matmul_pq(xq, xs, wq_f, ws_f, compute)
         ctx.save_for_backward(*saved_x, wq_d, ws_d)
         ctx.fp8_wgrad = fp8_wgrad
+        ctx.stage_major = stage_major
         ctx.pad_k = pad_k
         ctx.x_dtype = x.dtype
         ctx.compute = compute
@@ -91,10 +96,10 @@ class _MXFP8Linear(torch.autograd.Function):
         dx = dw = None
         padded = ctx.pad_k(d2d)
         if need_dw and ctx.fp8_wgrad:
-            dq, ds, dtq, dts = quantize_mx_dual(padded)
+            dq, ds, dtq, dts = quantize_mx_dual(padded, stage_major_t=ctx.stage_major)
             n = ctx.out_features
             # dW (out,in) = dY^T (out,tokens) . (X^T (in,tokens))^T, contraction over tokens.
-            wgrad = (dtq[:n], dts[:n], x_a, x_b)
+            wgrad = (dtq if ctx.stage_major else dtq[:n], dts[:n], x_a, x_b)
             if need_dx and ctx.x_dtype == ctx.compute:
                 # few tiles with a long K beside many with a short one: one launch shares the GPU
                 dx, dw = mxfp8_matmul_pq_batch([(dq, ds, wq_d, ws_d), wgrad], ctx.compute)

@@ -187,7 +187,10 @@ def mxfp8_matmul_pq(
 
     ``aq (M,K)``, ``bq (N,K)`` e4m3 and ``a_scale (M,K//32)``, ``b_scale (N,K//32)``
     ue8m0 in the natural layout ``quantize_mx`` produces.  Needs only ``K % 32 == 0``.
+    A 3-D ``(K // 128, rows, 128)`` code tensor is a stage-major operand (``quantize_mx_dual``).
     """
+    if aq.dim() == 3 or bq.dim() == 3:
+        return mxfp8_matmul_pq_batch([(aq, a_scale, bq, b_scale)], out_dtype)[0]
     if aq.dim() != 2 or bq.dim() != 2 or aq.shape[1] != bq.shape[1]:
         raise ValueError(f"contraction mismatch: {tuple(aq.shape)} @ {tuple(bq.shape)}.T")
     m, k = aq.shape
