@@ -344,6 +344,8 @@ int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, int64_t C, i
  * (stride_dwe, lddw) in elements.  An expert without rows gets zeros.  The MXFP8 form of
  * grouped_mxfp8_wgrad_kernel / _launch_wgrad (grouped.py:152-247, moe.py:64-99), which
  * multiply in 16 bits.
+ * When both scale pitches leave 12 readable bytes behind a row's last stage (ldas, ldbs >=
+ * mpad/32 + 12) the kernel fetches a row's scale bytes 16 at a time instead of 4.
  */
 int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t lda, int64_t ldas, const uint8_t *bq,
                         const uint8_t *bs, int64_t ldb, int64_t ldbs, const int32_t *offsets, int64_t E,

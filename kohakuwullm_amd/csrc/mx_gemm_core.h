@@ -184,8 +184,13 @@ __device__ __forceinline__ void issue_stage(const IssueCtx<S> &c, const Lane &L,
 
 // How a row's scale bytes are fetched: one 16-byte load per 512 of K (K % 512 == 0, 16-byte
 // aligned rows), one dword per stage (K % 128 == 0, 4-byte aligned rows), or byte by byte (any
-// K % 32 == 0 and any pitch; blocks past the end of K read as scale byte 0).
-enum { SCALES_VEC16 = 0, SCALES_DWORD = 1, SCALES_BYTES = 2 };
+// K % 32 == 0 and any pitch; blocks past the end of K read as scale byte 0).  SCALES_QUAD: one
+// 16-byte load per 4 stages from a 4-byte aligned address, for K ranges that start on any stage
+// (the token ranges of experts); it reads up to 12 bytes past the last stage's bytes, which the
+// caller guarantees to lie inside the row's pitch.  Against SCALES_DWORD it asks the L2 for a
+// row's line once per four stages instead of once per stage: 512 rows x 4 bytes a stage is half
+// as many lines again as the stage's codes.
+enum { SCALES_VEC16 = 0, SCALES_DWORD = 1, SCALES_BYTES = 2, SCALES_QUAD = 3 };
 
 // 16 scale bytes (4 stages x 4 blocks) of one row starting at scale column kb0.
 template <int MODE>
@@ -193,6 +198,10 @@ __device__ __forceinline__ void load_scales(const uint8_t *row, int kb0, int kb_
     const uint8_t *p = row + kb0;
     if (MODE == SCALES_VEC16) {
         v4i t = *(const v4i *)p;
+        d[0] = t[0], d[1] = t[1], d[2] = t[2], d[3] = t[3];
+    } else if (MODE == SCALES_QUAD) {
+        typedef int v4i_a4 __attribute__((ext_vector_type(4), aligned(4)));
+        v4i_a4 t = *(const v4i_a4 *)p;
         d[0] = t[0], d[1] = t[1], d[2] = t[2], d[3] = t[3];
     } else if (MODE == SCALES_DWORD) {
 #pragma unroll

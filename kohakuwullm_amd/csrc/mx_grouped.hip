@@ -972,14 +972,14 @@ __global__ __launch_bounds__(256) void wgrad_zero_kernel(WgradArgs p, int chunks
     }
 }
 
-template <typename S, int CDT>
+template <typename S, int CDT, int SCALES>
 __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     __shared__ ExpertTable table;
     const bool tabled = args.E <= MX_TABLE_MAX;
     if (tabled) build_live_table(table, args.offsets, args.E);
     WgradProblem<S, CDT> prob(args, tabled ? &table : nullptr);
-    persistent_gemm<S, SCALES_DWORD>(prob, smem);
+    persistent_gemm<S, SCALES>(prob, smem);
 }
 
 // Adds the K slices of every tile of every non-empty expert, in slice order, and stores dW.
@@ -1231,7 +1231,9 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
     a.ws = work < (1 << 27) ? mx::split_scratch(st, cus, (size_t)S::BM * S::BN) : nullptr;
     a.slots = a.ws ? 2 * cus : 0;
     dim3 grid((unsigned)(work * (a.slots ? 8 : 1) < cus ? work * (a.slots ? 8 : 1) : cus)), block(S::NTHR);
-    auto kern = grouped_wgrad_kernel<S, CDT>;
+    // scale rows with 12 readable bytes behind their last stage take one 16-byte fetch per four stages
+    const bool quad = a.ldas >= a.KB + 12 && a.ldbs >= a.KB + 12;
+    auto kern = quad ? grouped_wgrad_kernel<S, CDT, SCALES_QUAD> : grouped_wgrad_kernel<S, CDT, SCALES_DWORD>;
     if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     const int chunks = (a.N + 63) / 64;
     if ((int64_t)a.E * chunks >= 0x7FFFFFFF) return MX_EUNSUPPORTED;

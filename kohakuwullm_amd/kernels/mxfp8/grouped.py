@@ -19,6 +19,7 @@ from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE
 
 _FP8 = torch.float8_e4m3fn
 WGRAD_ROW_TILE = 128  # an expert's rows start on a multiple of this in the padded token axis
+SCALE_ROW_SLACK = 16  # spare bytes behind each token-axis scale row (see token_axis_buffers)
 
 
 def _check_offsets(offsets: torch.Tensor, num_experts: int) -> None:
@@ -112,7 +113,9 @@ def token_axis_buffers(cols: int, mpad: int, device):
     """``(cols, mpad)`` codes and ``(cols, mpad // 32)`` scales for a token-axis quantization, as views of wider rows."""
     pitch = mpad + TOKEN_PITCH_PAD
     qt = torch.empty(cols, pitch, device=device, dtype=_FP8)[:, :mpad]
-    st = torch.empty(cols, mpad // BLOCK_SCALE, device=device, dtype=torch.uint8)
+    # 16 spare bytes behind every scale row: the expert WGRAD then fetches a row's scales 16 bytes at a
+    # time from wherever an expert's token range starts (it may read 12 bytes past the row's last stage)
+    st = torch.empty(cols, mpad // BLOCK_SCALE + SCALE_ROW_SLACK, device=device, dtype=torch.uint8)[:, : mpad // BLOCK_SCALE]
     return qt, st
 
 

@@ -174,6 +174,11 @@ def test_grouped_token_axis_quantizer_and_wgrad(oracle, counts):
     # WGRAD on the token-axis operands: per-expert A^T B of the dequantized padded blocks
     dw = grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets.to(DEV), m)
     assert dw.shape == (e, n, k)
+    # the quantizer leaves spare bytes behind every scale row and the kernel then fetches scales 16 bytes
+    # at a time; scale rows packed end to end take the dword-per-stage path: same result, bit for bit
+    assert ats.stride(0) > ats.shape[1] and bts.stride(0) > bts.shape[1]
+    dw_packed = grouped_mxfp8_wgrad(atq, ats.contiguous(), btq, bts.contiguous(), offsets.to(DEV), m)
+    assert torch.equal(dw, dw_packed)
     ad = oracle.dequant(rq.T.contiguous().T, rs)  # (n, mpad)
     bd = oracle.dequant(bq_ref, bs_ref)  # (k, mpad)
     pos = 0
