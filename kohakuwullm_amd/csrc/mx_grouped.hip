@@ -174,7 +174,8 @@ __device__ __forceinline__ void build_row_tile_table(ExpertTable &tb, const int3
     __syncthreads();
 }
 
-// a[j] = the j-th expert with rows, b[j] = 128-token K stages of the experts before it; n = how many.
+// a[j] = the j-th expert with rows, b[j] = 128-token K stages of the experts before it; n = how many;
+// b[n] = K stages of all experts.
 __device__ __forceinline__ void build_live_table(ExpertTable &tb, const int32_t *__restrict__ offsets, int E) {
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
@@ -194,7 +195,10 @@ __device__ __forceinline__ void build_live_table(ExpertTable &tb, const int32_t 
             carry_l += __builtin_popcountll(mask);
             carry_p += __shfl(ip, 63, 64);
         }
-        if (lane == 0) tb.n = carry_l;
+        if (lane == 0) {
+            tb.n = carry_l;
+            tb.b[carry_l] = carry_p;  // one past the last expert's K stages
+        }
     }
     __syncthreads();
 }
@@ -800,6 +804,32 @@ struct WgradArgs {
     int slots;
 };
 
+// Even K split (needs the LDS table of the experts with rows).  The K stages of those experts,
+// laid end to end, are cut into G / tiles_per_expert equal ranges of `q` stages; a group of
+// tiles_per_expert workgroups, one per output tile, takes each range.  A range that covers an
+// expert's stages only in part leaves fp32 partial sums: at most two per workgroup (the end of
+// an expert an earlier group began, the beginning of one a later group ends), in slots 2 u and
+// 2 u + 1 of workgroup-unit u, and wgrad_reduce_kernel adds an expert's pieces in group order.
+// Every workgroup works one range of equal length, where whole K slices left a ragged second
+// round and one fp32 partial tile per slice (measured at six busy experts of 16384 rows:
+// 480 partial tiles and two rounds against 336 and one).
+struct WgradEven {
+    int per_e, groups, q, total;
+};
+
+__device__ __forceinline__ WgradEven wgrad_even_plan(const WgradArgs &p, int workgroups, const ExpertTable &tb) {
+    WgradEven v;
+    v.per_e = p.tiles_m * p.tiles_n;
+    v.groups = workgroups / v.per_e;  // > 0: the split is only chosen when the tiles leave workgroups idle
+    v.total = tb.b[tb.n];
+    v.q = (v.total + v.groups - 1) / v.groups;
+    return v;
+}
+
+// The workgroups of one XCD (b % 8) take consecutive unit numbers, so that the tiles of one
+// (expert, K range), which read the same operand panels, share that XCD's L2.
+__device__ __forceinline__ int wgrad_unit_of(int b, int g) { return (g & 7) == 0 ? (b & 7) * (g >> 3) + (b >> 3) : b; }
+
 // Number of K slices per tile: as many as fill the GPU about twice over, at most 8, and 1 when
 // the tiles of the non-empty experts already fill three quarters of it.  Also counts the
 // non-empty experts.
@@ -832,6 +862,10 @@ struct WgradProblem {
     // incremental scan: expert scan_e is the scan_live-th non-empty one and its first K stage
     // is scan_tiles
     int scan_e, scan_tiles, scan_live;
+    // even K split: this workgroup's unit number, its remaining range of K stages, the split's plan
+    bool even;
+    int unit, pos, end;
+    WgradEven ev;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
 
     // Workgroups are dealt to the 8 XCDs round-robin, so workgroup b starts at unit
@@ -843,8 +877,17 @@ struct WgradProblem {
     __device__ WgradProblem(const WgradArgs &a, const ExpertTable *table)
         : p(a), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0), tb(table) {
         const int g = (int)gridDim.x, b = (int)blockIdx.x;
-        next_unit = (g & 7) == 0 ? (b & 7) * (g >> 3) + (b >> 3) : b;
+        next_unit = wgrad_unit_of(b, g);
         slices = wgrad_slices(p, g, live, tb);
+        even = tb && slices > 1;
+        if (even) {
+            ev = wgrad_even_plan(p, g, *tb);
+            unit = next_unit;
+            const int grp = unit / ev.per_e;
+            pos = grp < ev.groups ? grp * ev.q : ev.total;
+            pos = pos < ev.total ? pos : ev.total;
+            end = pos + ev.q < ev.total ? pos + ev.q : ev.total;
+        }
     }
 
     __device__ __forceinline__ void zero_slot(int slot) const {
@@ -854,6 +897,26 @@ struct WgradProblem {
 
     __device__ __forceinline__ bool next(Tile &t) {
         const int per_e = p.tiles_m * p.tiles_n;
+        if (even) {
+            if (pos >= end) return false;
+            // the expert whose K stages hold `pos`: the last j with b[j] <= pos
+            int lo = 0, hi = tb->n - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (tb->b[mid] <= pos) lo = mid;
+                else hi = mid - 1;
+            }
+            const int first = tb->b[lo], past = tb->b[lo + 1];
+            const int rem = unit % per_e;
+            t.expert = tb->a[lo];
+            t.m0 = (rem / p.tiles_n) * S::BM;
+            t.n0 = (rem % p.tiles_n) * S::BN;
+            t.kt0 = pos;
+            t.kt1 = end < past ? end : past;
+            t.slot = (t.kt0 == first && t.kt1 == past) ? -1 : 2 * unit + (t.kt0 > first ? 0 : 1);
+            pos = t.kt1;
+            return true;
+        }
         const int per_live = per_e * slices;
         while (next_unit < live * per_live) {
             const int unit = next_unit;
@@ -1015,10 +1078,22 @@ __global__ __launch_bounds__(S::NTHR) void wgrad_reduce_kernel(WgradArgs p, int 
         v4f sum[S::NT];
 #pragma unroll
         for (int jj = 0; jj < S::NT; jj++) sum[jj] = v4f{0.f, 0.f, 0.f, 0.f};
-        for (int sl = 0; sl < slices; sl++) {
-            const v4f *src = (const v4f *)p.ws + (int64_t)((j * per_e + rem) * slices + sl) * (S::BM * S::BN / 4);
+        if (tabled) {  // even K split: the pieces of the groups whose ranges meet this expert's stages
+            const WgradEven ev = wgrad_even_plan(p, workgroups, table);
+            const int g_lo = table.b[j] / ev.q, g_hi = (table.b[j + 1] - 1) / ev.q;
+            if (g_lo == g_hi) continue;  // one group had all of it and stored the tile itself
+            for (int g = g_lo; g <= g_hi; g++) {
+                const int slot = 2 * (g * per_e + rem) + (g == g_lo ? 1 : 0);
+                const v4f *src = (const v4f *)p.ws + (int64_t)slot * (S::BM * S::BN / 4);
 #pragma unroll
-            for (int jj = 0; jj < S::NT; jj++) sum[jj] += src[(i * S::NT + jj) * S::NTHR + tid];
+                for (int jj = 0; jj < S::NT; jj++) sum[jj] += src[(i * S::NT + jj) * S::NTHR + tid];
+            }
+        } else {
+            for (int sl = 0; sl < slices; sl++) {
+                const v4f *src = (const v4f *)p.ws + (int64_t)((j * per_e + rem) * slices + sl) * (S::BM * S::BN / 4);
+#pragma unroll
+                for (int jj = 0; jj < S::NT; jj++) sum[jj] += src[(i * S::NT + jj) * S::NTHR + tid];
+            }
         }
         const int n = (rem % p.tiles_n) * S::BN + wn * S::WTN + 8 * (lane & 15);
 #pragma unroll

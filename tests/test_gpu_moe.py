@@ -192,6 +192,38 @@ def test_grouped_token_axis_quantizer_and_wgrad(oracle, counts):
             assert oracle.rel_error(dw[i].cpu(), ref) < TOL, (i, cnt)
 
 
+@pytest.mark.parametrize("counts", [[2400, 0, 700, 2900], [5000, 1], [130, 0, 0, 4000, 0, 1500]])
+def test_wgrad_even_k_split_ranges_straddle_experts(oracle, counts):
+    """Few busy experts with several output tiles each: the K stages of all experts are cut into equal
+    ranges, one per group of workgroups, and ranges end inside an expert and straddle two of them
+    (19 + 6 + 23 stages in ranges of 2, for the first case).  Every expert against the fp64 oracle."""
+    from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_wgrad, quantize_mx_cols_grouped
+
+    g = torch.Generator().manual_seed(SEED + 7)
+    e, m = len(counts), sum(counts)
+    n, k = 512, 384  # 2 x 2 output tiles per expert
+    offsets = torch.zeros(e + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    a = (torch.randn(m, n, generator=g) * 1e-2).bfloat16()
+    b = torch.randn(m, k, generator=g).bfloat16()
+    atq, ats = quantize_mx_cols_grouped(a.to(DEV), offsets.to(DEV), m)
+    btq, bts = quantize_mx_cols_grouped(b.to(DEV), offsets.to(DEV), m)
+    dw = grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets.to(DEV), m)
+    assert torch.equal(dw, grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets.to(DEV), m))  # deterministic
+    aq_ref, as_ref, _ = _padded_cols_ref(oracle, a.float(), offsets)
+    bq_ref, bs_ref, _ = _padded_cols_ref(oracle, b.float(), offsets)
+    ad, bd = oracle.dequant(aq_ref, as_ref), oracle.dequant(bq_ref, bs_ref)
+    pos = 0
+    for i, cnt in enumerate(counts):
+        tiles = -(-cnt // 128)
+        ref = ad[:, pos : pos + tiles * 128] @ bd[:, pos : pos + tiles * 128].T
+        pos += tiles * 128
+        if cnt == 0:
+            assert (dw[i] == 0).all()
+        else:
+            assert oracle.rel_error(dw[i].cpu(), ref) < TOL, (i, cnt)
+
+
 def _expert_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
     """The fused path's arithmetic restated with oracle primitives, stage by stage."""
     e, two_h, dim = w_in.shape
