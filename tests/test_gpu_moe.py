@@ -192,6 +192,33 @@ def test_grouped_token_axis_quantizer_and_wgrad(oracle, counts):
             assert oracle.rel_error(dw[i].cpu(), ref) < TOL, (i, cnt)
 
 
+@pytest.mark.parametrize("with_scale", [False, True])
+def test_grouped_token_axis_quantizer_many_rows(oracle, with_scale):
+    """Enough routed rows and columns that a workgroup walks four column tiles of its 128 rows
+    (the launch picks that for 512 or more row tiles of 4 or more column tiles): bit-exact."""
+    from kohakuwullm_amd.kernels.mxfp8.grouped import quantize_mx_cols_grouped
+
+    g = torch.Generator().manual_seed(SEED + 11)
+    counts = [30000, 0, 20001, 17000, 130]
+    e, m = len(counts), sum(counts)
+    tokens, c = 4096, 640  # five column tiles: one workgroup of four, one of one
+    offsets = torch.zeros(e + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    x = torch.randn(tokens, c, generator=g).bfloat16()
+    index = torch.randint(0, tokens, (m,), generator=g).int()
+    scale = (torch.rand(m, generator=g) + 0.5).bfloat16()
+    sidx = torch.randperm(m, generator=g).int()
+    kw = dict(row_scale=scale.to(DEV), scale_index=sidx.to(DEV)) if with_scale else {}
+    tq, ts = quantize_mx_cols_grouped(x.to(DEV), offsets.to(DEV), m, index=index.to(DEV), **kw)
+    rows = x[index.long()].float()
+    if with_scale:
+        rows = rows * scale[sidx.long()].float()[:, None]
+    rq, rs, valid = _padded_cols_ref(oracle, rows, offsets)
+    vs = valid.view(-1, 32)[:, 0]
+    assert torch.equal(tq.view(torch.uint8).cpu()[:, valid], rq[:, valid])
+    assert torch.equal(ts.cpu()[:, vs], rs[:, vs])
+
+
 @pytest.mark.parametrize("counts", [[2400, 0, 700, 2900], [5000, 1], [130, 0, 0, 4000, 0, 1500]])
 def test_wgrad_even_k_split_ranges_straddle_experts(oracle, counts):
     """Few busy experts with several output tiles each: the K stages of all experts are cut into equal
