@@ -137,6 +137,7 @@ struct DenseProblem {
     }
 
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
+    static constexpr bool EARLY_WAIT = false;  // interior tiles leave exactly NST stores in flight instead
 
     // Slot of workgroup `wg`'s piece of the split tile whose stages start at `begin` in the
     // split stage space: a workgroup has at most two partial units, the first one continuing

@@ -330,6 +330,7 @@ struct LdsScratch {
 //                                           lane issued if that number is the same compile-time
 //                                           constant P::NST for the whole wave, else -1
 //   int  P::kb_end                          scale bytes per row (bound for predicated fetches)
+//   bool P::EARLY_WAIT                      wait for the next tile's first stage before the epilogue (see the tile loop)
 template <typename S, int K512, typename P>  // K512: one of SCALES_*
 __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     uint8_t *const ldsA = smem;                                                  // [2][BM*128]
@@ -437,15 +438,28 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         // of stores the wait lets exactly those stay in flight,
         // so the stores drain under the next tile's first stage.
         const int lastbuf = (gstage - 1) & 1;
+        // P::EARLY_WAIT (epilogues whose lanes issue differing numbers of stores, so that no count of
+        // them can be left in flight behind the next tile's copies): the wait for those copies and for
+        // the next tile's scale bytes comes BEFORE the epilogue, where only they are outstanding, the
+        // scales are parked then (their planes were last read two super-steps ago, with a barrier
+        // since), and the barrier behind the epilogue publishes both.  The epilogue's own stores then
+        // need no wait at all and drain under the next tile's K loop instead of in front of it.
+        if (P::EARLY_WAIT && has_next) {
+            wait_vm_allow_c<0>();
+            if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
+            if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);
+        }
         const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B,
                                             (uint8_t *)(ldsSA + ((gsuper - 1) & 1) * 4 * S::PA)});
-        if (has_next) {
+        if (!P::EARLY_WAIT && has_next) {
             if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
             if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);
         }
         if (!has_next) break;
-        if (stores == P::NST) wait_vm_allow_c<P::NST>();
-        else wait_vm_allow_c<0>();
+        if (!P::EARLY_WAIT) {
+            if (stores == P::NST) wait_vm_allow_c<P::NST>();
+            else wait_vm_allow_c<0>();
+        }
         __syncthreads();
         cur = nxt;
         has_next = prob.next(nxt);

@@ -223,6 +223,8 @@ struct GroupedProblem {
     // units and a lane owns 4 consecutive ones, gate and value.
     static constexpr int N_PER_TILE = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
+    // the fused epilogues issue a different number of stores per lane (row and column masks): see persistent_gemm
+    static constexpr bool EARLY_WAIT = MODE == MODE_GEMM1 || MODE == MODE_DGRAD2;
 
     const ExpertTable *tb;  // row-tile prefix table in LDS, or nullptr (more experts than it holds)
 
@@ -623,6 +625,14 @@ struct GroupedProblem {
 
         __syncthreads();  // every wave is out of the main loop: the stage buffer is free
         const int64_t pbase = t.ppos;
+        // Lane-dependent offsets of the passes below are derived from an opaque copy of the lane id.
+        // From the plain one they are invariants of the tile loop: the compiler computed them once,
+        // could not keep them in registers across the main loop, and reloaded each from scratch
+        // memory right before its use behind a full vector-memory wait, which also waited for the
+        // pass's previous global store: the stores of a pass went out one round trip at a time
+        // (127 reloads per tile; C4: 235 -> 224 us).
+        const Lane Lo = opaque(L);
+        const int o_tid = Lo.tid, o_r16 = Lo.lane & 15, o_g = Lo.lane >> 4;
 #pragma unroll
         for (int pass = 0; pass < 4; pass++) {
             // pass = (gate | value, low | high four of the lane's eight columns); staged column
@@ -653,15 +663,15 @@ struct GroupedProblem {
                     cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
                     const uint32_t byte = scale_byte(cm);
                     const float inv = inv_scale(byte);
-                    const int col = L.wn * (S::WTN / 2) + 4 * L.r16 + e;
+                    const int col = L.wn * (S::WTN / 2) + 4 * o_r16 + e;
 #pragma unroll
                     for (int ii = 0; ii < 2; ii++) {
-                        const int row = L.wm * S::WTM + 16 * (2 * blk + ii) + 4 * L.g;  // 4 consecutive rows: one dword
+                        const int row = L.wm * S::WTM + 16 * (2 * blk + ii) + 4 * o_g;  // 4 consecutive rows: one dword
                         const uint32_t w = pack4_e4m3(val[ii][0] * inv, val[ii][1] * inv, val[ii][2] * inv, val[ii][3] * inv);
                         // column-major, 256 bytes per column, 16-byte chunks XOR-swizzled by the lane's r16
                         *(uint32_t *)(codes + col * S::BM + ((((row >> 4) ^ (col >> 2)) & 15) << 4) + (row & 15)) = w;
                     }
-                    if (L.g == 0) bytes[col * (S::BM / 32) + L.wm * (S::WTM / 32) + blk] = (uint8_t)byte;
+                    if (o_g == 0) bytes[col * (S::BM / 32) + L.wm * (S::WTM / 32) + blk] = (uint8_t)byte;
                 }
             }
             __syncthreads();
@@ -669,7 +679,7 @@ struct GroupedProblem {
             // that starts past the expert's rows belongs to the next expert's padding and is skipped
 #pragma unroll
             for (int k = 0; k < (S::BN / 2) * S::BM / 16 / S::NTHR; k++) {
-                const int q = L.tid + k * S::NTHR;
+                const int q = o_tid + k * S::NTHR;
                 const int col = q >> 4, ch = q & 15;
                 const int hcol = t.n0 + 8 * (col >> 2) + 4 * sub + (col & 3);
                 const bool half_ok = t.row0 + (ch >> 3) * 128 < t.end;
@@ -678,10 +688,10 @@ struct GroupedProblem {
                     *(v4i *)(p.htq + (int64_t)(half * H + hcol) * p.ldhtq + pbase + ch * 16) = w;
                 }
             }
-            if (L.tid < S::BN / 2) {
-                const int hcol = t.n0 + 8 * (L.tid >> 2) + 4 * sub + (L.tid & 3);
+            if (o_tid < S::BN / 2) {
+                const int hcol = t.n0 + 8 * (o_tid >> 2) + 4 * sub + (o_tid & 3);
                 if (hcol < H) {
-                    const uint32_t *src = (const uint32_t *)(bytes + L.tid * (S::BM / 32));
+                    const uint32_t *src = (const uint32_t *)(bytes + o_tid * (S::BM / 32));
                     uint8_t *dst = p.hts + (int64_t)(half * H + hcol) * p.ldhts + (pbase >> 5);
                     *(uint32_t *)dst = src[0];
                     if (t.row0 + 128 < t.end) *(uint32_t *)(dst + 4) = src[1];
@@ -867,6 +877,7 @@ struct WgradProblem {
     int unit, pos, end;
     WgradEven ev;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
+    static constexpr bool EARLY_WAIT = false;
 
     // Workgroups are dealt to the 8 XCDs round-robin, so workgroup b starts at unit
     // (b % 8) * (G / 8) + b / 8: the workgroups of one XCD take consecutive units, i.e. the tiles
