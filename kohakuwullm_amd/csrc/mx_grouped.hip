@@ -458,10 +458,13 @@ struct GroupedProblem {
         __syncthreads();
         // 16 consecutive lanes write the 256 bytes of one hidden unit's 256 tokens; a 128-row half
         // that starts past the expert's rows belongs to the next expert's padding and is skipped
-        const int64_t pbase = t.ppos;
+        // wave-uniform and lane-dependent parts of the addresses below are rebuilt here (scalar register,
+        // opaque lane id): as invariants of the tile loop they were spilled and reloaded behind full waits
+        const int64_t pbase = __builtin_amdgcn_readfirstlane(t.ppos);
+        const int o_tid = opaque(L).tid;
 #pragma unroll
         for (int k = 0; k < N_PER_TILE * S::BM / 16 / S::NTHR; k++) {
-            const int q = L.tid + k * S::NTHR;
+            const int q = o_tid + k * S::NTHR;
             const int col = q >> 4, ch = q & 15;
             const bool half_ok = t.row0 + (ch >> 3) * 128 < t.end;
             if (t.n0 + col < p.N && half_ok) {
@@ -469,9 +472,9 @@ struct GroupedProblem {
                 *(v4i *)(p.htq + (int64_t)(t.n0 + col) * p.ldhtq + pbase + ch * 16) = w;
             }
         }
-        if (L.tid < N_PER_TILE && t.n0 + L.tid < p.N) {
-            const uint32_t *src = (const uint32_t *)(lds.b + L.tid * (S::BM / 32));
-            uint8_t *dst = p.hts + (int64_t)(t.n0 + L.tid) * p.ldhts + (pbase >> 5);
+        if (o_tid < N_PER_TILE && t.n0 + o_tid < p.N) {
+            const uint32_t *src = (const uint32_t *)(lds.b + o_tid * (S::BM / 32));
+            uint8_t *dst = p.hts + (int64_t)(t.n0 + o_tid) * p.ldhts + (pbase >> 5);
             *(uint32_t *)dst = src[0];
             if (t.row0 + 128 < t.end) *(uint32_t *)(dst + 4) = src[1];
         }
@@ -624,7 +627,7 @@ struct GroupedProblem {
         if (!tok) return -1;
 
         __syncthreads();  // every wave is out of the main loop: the stage buffer is free
-        const int64_t pbase = t.ppos;
+        const int64_t pbase = __builtin_amdgcn_readfirstlane(t.ppos);
         // Lane-dependent offsets of the passes below are derived from an opaque copy of the lane id.
         // From the plain one they are invariants of the tile loop: the compiler computed them once,
         // could not keep them in registers across the main loop, and reloaded each from scratch
