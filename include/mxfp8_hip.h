@@ -292,7 +292,10 @@ int mx_experts_scatter_gemm(const uint8_t *aq, const uint8_t *as, int64_t a_rows
  * output of mx_grouped_gemm_nt), pair t*top_k + k sits at the sorted position m with
  * order[m] == t*top_k + k and m < offsets[E] (a pair found nowhere was dropped and adds
  * nothing), and scale = gate[pair] (NULL: 1).  fp32 sum in k order, one rounding: one writer
- * per element, bitwise reproducible.  `inv` is caller-provided scratch of T*top_k int32.
+ * per element, bitwise reproducible.  `inv` is caller-provided scratch of T*top_k int32: the call
+ * fills it with pos(t,k) (-1 for a dropped pair).  With order == NULL the call takes inv as filled
+ * by an earlier call for the same routing and skips that step (a layer's backward reuses its
+ * forward's).
  * Every element of out is written; out need not be zeroed.
  * Stands in for the tl.atomic_add epilogues of _experts_gemm2 (experts.py:138-222) and
  * _experts_gemm1_dgrad (experts_bwd.py:167-247) when order is the reference's pair index

@@ -1281,7 +1281,7 @@ extern "C" int mx_experts_combine(const void *y, int64_t ldy, const int32_t *ord
                                   const void *gate, int gate_dtype, int32_t *inv, int64_t T, int64_t top_k, void *out,
                                   int dtype, int64_t ldo, int64_t M, int64_t N, void *stream) {
     if (E <= 0 || E >= (1 << 20) || T < 0 || top_k <= 0 || top_k > 0x7FFF || M < 0 || N < 0 || M >= 0x7FFFFFFF ||
-        T * top_k >= 0x7FFFFFFF || ldy < N || ldo < N || !order || !offsets || !inv)
+        T * top_k >= 0x7FFFFFFF || ldy < N || ldo < N || (order && !offsets) || !inv)
         return MX_EINVAL;
     if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EINVAL;
     if (gate && gate_dtype != MX_FP32 && gate_dtype != dtype) return MX_EINVAL;
@@ -1289,8 +1289,10 @@ extern "C" int mx_experts_combine(const void *y, int64_t ldy, const int32_t *ord
     if (N % 8 || !aligned(y, 16) || !aligned(out, 16) || ldy % 8 || ldo % 8) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
     const int64_t pairs = T * top_k;
-    fill_i32_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>(inv, pairs, -1);
-    if (M) invert_order_kernel<<<dim3((unsigned)((M + 255) / 256)), dim3(256), 0, st>>>(order, offsets, (int)E, M, pairs, inv);
+    if (order) {  // order == NULL: inv already holds the positions of this routing (an earlier call filled it)
+        fill_i32_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>(inv, pairs, -1);
+        if (M) invert_order_kernel<<<dim3((unsigned)((M + 255) / 256)), dim3(256), 0, st>>>(order, offsets, (int)E, M, pairs, inv);
+    }
     const int n8 = (int)(N / 8);
     const int64_t blocks = (T * n8 + 255) / 256;
     if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;

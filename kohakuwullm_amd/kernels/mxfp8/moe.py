@@ -131,25 +131,32 @@ def launch_scatter_gemm(aq, a_s, wq, ws, out, token_of, order, gate, offsets, in
     )
 
 
-def combine_sorted_rows(y, order, offsets, num_experts, gate, tokens: int, top_k: int) -> torch.Tensor:
+def combine_sorted_rows(y, order, offsets, num_experts, gate, tokens: int, top_k: int, positions=None,
+                        return_positions: bool = False):
     """``out[t] = sum_k gate[t*top_k+k] * y[position of pair t*top_k+k]``: the scatter-add as a gather.
 
     ``order`` must be the pair index ``token * top_k + slot`` (what ``expert_sort`` produces).
-    Deterministic; every row of the result is written.
+    Deterministic; every row of the result is written.  ``positions``: the pair -> sorted position
+    table an earlier call for the same routing returned (``return_positions=True``); with it the
+    call skips rebuilding the table from ``order``.
     """
     m, n = y.shape
     out = torch.empty(tokens, n, device=y.device, dtype=y.dtype)
-    inv = torch.empty(tokens * top_k, device=y.device, dtype=torch.int32)
+    reuse = positions is not None
+    if reuse and (positions.numel() != tokens * top_k or positions.dtype != torch.int32 or positions.device != y.device):
+        raise ValueError(f"positions {tuple(positions.shape)} {positions.dtype} does not fit {tokens} tokens x top_k {top_k}")
+    inv = positions if reuse else torch.empty(tokens * top_k, device=y.device, dtype=torch.int32)
     _lib.invoke(
         "mx_experts_combine", y.element_size() * n * (tokens * top_k + tokens), y,
-        y.data_ptr(), y.stride(0), order.data_ptr(), offsets.data_ptr(), num_experts,
+        y.data_ptr(), y.stride(0), 0 if reuse else order.data_ptr(), offsets.data_ptr(), num_experts,
         0 if gate is None else gate.data_ptr(), 0 if gate is None else _lib.MX_DTYPE[gate.dtype], inv.data_ptr(),
         tokens, top_k, out.data_ptr(), _lib.MX_DTYPE[out.dtype], out.stride(0), m, n,
     )
-    return out
+    return (out, inv) if return_positions else out
 
 
-def _routed_product(aq, a_s, wq, ws, token_of, order, gate, offsets, tokens: int, top_k: int, dtype) -> torch.Tensor:
+def _routed_product(aq, a_s, wq, ws, token_of, order, gate, offsets, tokens: int, top_k: int, dtype, positions=None,
+                    return_positions: bool = False):
     """``out[token] += scale * (a[m] . w[e(m)]^T)`` over the sorted rows.
 
     When ``order`` is a pair index (``top_k`` > 0) the rows are written once by the grouped GEMM
@@ -159,10 +166,10 @@ def _routed_product(aq, a_s, wq, ws, token_of, order, gate, offsets, tokens: int
     n = wq.shape[1]
     if top_k > 0 and n % 8 == 0:
         y = grouped_mxfp8_gemm(aq, a_s, wq, ws, offsets, out_dtype=dtype, rows=token_of.numel())
-        return combine_sorted_rows(y, order, offsets, wq.shape[0], gate, tokens, top_k)
+        return combine_sorted_rows(y, order, offsets, wq.shape[0], gate, tokens, top_k, positions, return_positions)
     out = torch.zeros(tokens, n, device=aq.device, dtype=dtype)
     launch_scatter_gemm(aq, a_s, wq, ws, out, token_of, order if gate is not None else None, gate, offsets)
-    return out
+    return (out, None) if return_positions else out
 
 
 def launch_gemm2_dgrad(dq, ds, token_of, order, gate, wq, ws, hq, hs, pre, dpre, dpq, dps, dgate, offsets,
@@ -207,8 +214,11 @@ class _MXFP8Experts(torch.autograd.Function):
         launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hidden, dim, x.dtype, htq, hts)
         # pairs per token when `order` is the pair index token * top_k + slot; 0 = unknown layout
         top_k = gate.numel() // rows if rows and gate.numel() % rows == 0 else 0
-        out = _routed_product(hq, hs, *packed.out_fwd, token_of, order, gate, offsets, rows, top_k, x.dtype)
+        # the pair -> sorted position table of the combine serves the backward's combine too
+        out, positions = _routed_product(hq, hs, *packed.out_fwd, token_of, order, gate, offsets, rows, top_k, x.dtype,
+                                         return_positions=True)
         if needs_grad:
+            ctx.positions = positions
             ctx.save_for_backward(x, hq, hs, pre, gate, token_of, order, offsets, htq, hts)
             ctx.packed = packed
             ctx.shapes = (hidden, dim, m, rows, top_k)
@@ -234,7 +244,8 @@ class _MXFP8Experts(torch.autograd.Function):
         dpre = None if ptq is not None else torch.empty(m, 2 * hidden, device=dev, dtype=dout.dtype)
         launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets,
                            ptq, pts)
-        dx = _routed_product(dpq, dps, *packed.in_dgrad, token_of, order, None, offsets, rows, top_k, dout.dtype)
+        dx = _routed_product(dpq, dps, *packed.in_dgrad, token_of, order, None, offsets, rows, top_k, dout.dtype,
+                             positions=ctx.positions)
 
         dw_in = dw_out = None
         if ctx.needs_input_grad[2]:

@@ -121,3 +121,11 @@ def test_expert_combine_direct(oracle):
                 for _ in range(2)]
         assert torch.equal(outs[0], outs[1]) and outs[0].dtype == torch.bfloat16
         assert oracle.rel_error(outs[0].cpu(), want) < 4e-3  # one bf16 rounding of an fp32 sum
+        # the pair -> position table of one call serves a later call for the same routing
+        gd = None if gt is None else gt.to(DEV)
+        out_a, pos = combine_sorted_rows(y.to(DEV), order.to(DEV), offsets.to(DEV), e, gd, tokens, top_k, return_positions=True)
+        out_b = combine_sorted_rows(y.to(DEV), None, offsets.to(DEV), e, gd, tokens, top_k, positions=pos)
+        assert torch.equal(out_a, outs[0]) and torch.equal(out_b, outs[0])
+        inv = pos.cpu()
+        assert torch.equal(inv[order[:m_real].long()], torch.arange(m_real, dtype=torch.int32))
+        assert (inv[order[m_real:].long()] == -1).all()
