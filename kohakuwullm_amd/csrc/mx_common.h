@@ -62,6 +62,16 @@ struct Elem<MX_BF16> {
         }
     }
     static __device__ __forceinline__ float load1(const void *p) { return bits2f((uint32_t)(*(const uint16_t *)p) << 16); }
+    // The same load in two halves, so that a kernel can put many of them in flight before it converts any.
+    typedef v4i raw;
+    static __device__ __forceinline__ raw load_raw(const void *p) { return *(const v4i *)p; }
+    static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = bits2f((uint32_t)r[i] << 16);
+            v[2 * i + 1] = bits2f((uint32_t)r[i] & 0xFFFF0000u);
+        }
+    }
 };
 
 template <>
@@ -74,6 +84,12 @@ struct Elem<MX_FP16> {
         for (int i = 0; i < 8; i++) v[i] = (float)r[i];
     }
     static __device__ __forceinline__ float load1(const void *p) { return (float)(*(const _Float16 *)p); }
+    typedef _Float16 raw __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ raw load_raw(const void *p) { return *(const raw *)p; }
+    static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (float)r[i];
+    }
 };
 
 template <>
@@ -88,6 +104,17 @@ struct Elem<MX_FP32> {
         }
     }
     static __device__ __forceinline__ float load1(const void *p) { return *(const float *)p; }
+    struct raw {
+        v4f a, b;
+    };
+    static __device__ __forceinline__ raw load_raw(const void *p) { return raw{((const v4f *)p)[0], ((const v4f *)p)[1]}; }
+    static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[i] = r.a[i];
+            v[4 + i] = r.b[i];
+        }
+    }
 };
 
 __device__ __forceinline__ float amax8(const float v[8]) {

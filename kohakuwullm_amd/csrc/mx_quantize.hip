@@ -300,10 +300,16 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict_
     const int64_t row0 = m0 + (t >> 4) * 8;
     const bool ok = col < K && m0 + (t >> 6) * 32 < M;  // K % 8 == 0 and M % 32 == 0
     float v[8][8];
+    // the thread's eight loads go out together (row by row, each waited for the one before it)
+    typename Elem<DT>::raw r[8];
+    if (ok) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) r[i] = Elem<DT>::load_raw((const T *)x + (row0 + i) * ldx + col);
+    }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         if (ok) {
-            Elem<DT>::load8((const T *)x + (row0 + i) * ldx + col, v[i]);
+            Elem<DT>::unpack(r[i], v[i]);
         } else {
 #pragma unroll
             for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
@@ -342,10 +348,15 @@ __global__ __launch_bounds__(256) void quant_dual_batch_kernel(QuantBatchArgs b)
     const int64_t row0 = m0 + (t >> 4) * 8;
     const bool ok = col < K && m0 + (t >> 6) * 32 < M;
     float v[8][8];
+    typename Elem<DT>::raw r[8];  // eight loads in flight, then the conversions
+    if (ok) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) r[i] = Elem<DT>::load_raw((const T *)x + (row0 + i) * ldx + col);
+    }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         if (ok) {
-            Elem<DT>::load8((const T *)x + (row0 + i) * ldx + col, v[i]);
+            Elem<DT>::unpack(r[i], v[i]);
         } else {
 #pragma unroll
             for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
@@ -370,12 +381,20 @@ __global__ __launch_bounds__(256) void swiglu_quant_dual_kernel(const void *__re
     const int64_t row0 = m0 + (t >> 4) * 8;
     const bool ok = col < H && m0 + (t >> 6) * 32 < M;
     float v[8][8];
+    typename Elem<DT>::raw rg[8], ru[8];  // all 16 loads in flight before the first conversion
+    if (ok) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            rg[i] = Elem<DT>::load_raw((const T *)gu + (row0 + i) * ldgu + col);
+            ru[i] = Elem<DT>::load_raw((const T *)gu + (row0 + i) * ldgu + H + col);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         if (ok) {
             float g[8], u[8];
-            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + col, g);
-            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + H + col, u);
+            Elem<DT>::unpack(rg[i], g);
+            Elem<DT>::unpack(ru[i], u);
 #pragma unroll
             for (int c = 0; c < 8; c++) v[i][c] = g[c] * sigmoid_fast(g[c]) * u[c];
         } else {
@@ -405,13 +424,25 @@ __global__ __launch_bounds__(256) void swiglu_bwd_quant_dual_kernel(const void *
     const int64_t row0 = m0 + (t >> 4) * 8;
     const bool ok = col < H && m0 + (t >> 6) * 32 < M;
     float v[8][8], w[8][8];
+    // All 24 loads of the thread go out before the first conversion.  Written row by row (load three,
+    // convert, next row) the compiler kept that order and every thread had 48 bytes in flight at a time,
+    // with a memory latency in front of each of its eight rows.
+    typename Elem<DT>::raw rg[8], ru[8], rd[8];
+    if (ok) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            rg[i] = Elem<DT>::load_raw((const T *)gu + (row0 + i) * ldgu + col);
+            ru[i] = Elem<DT>::load_raw((const T *)gu + (row0 + i) * ldgu + H + col);
+            rd[i] = Elem<DT>::load_raw((const T *)dh + (row0 + i) * lddh + col);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         if (ok) {
             float g[8], u[8], d[8];
-            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + col, g);
-            Elem<DT>::load8((const T *)gu + (row0 + i) * ldgu + H + col, u);
-            Elem<DT>::load8((const T *)dh + (row0 + i) * lddh + col, d);
+            Elem<DT>::unpack(rg[i], g);
+            Elem<DT>::unpack(ru[i], u);
+            Elem<DT>::unpack(rd[i], d);
 #pragma unroll
             for (int c = 0; c < 8; c++) {
                 float sg = sigmoid_fast(g[c]);
@@ -649,11 +680,17 @@ __global__ __launch_bounds__(256) void quant_cols_grouped_walk_kernel(GroupedQua
         const int64_t col = k0 + (t & 15) * 8;
         const bool col_ok = col < a.C;
         float v[8][8];
+        typename Elem<DT>::raw r[8];  // the eight row loads of this column tile go out together
+        if (SRC == SRC_PLAIN) {
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (col_ok && src[i] >= 0) r[i] = Elem<DT>::load_raw((const T *)a.x + src[i] * a.ldx + col);
+        }
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             if (col_ok && src[i] >= 0) {
                 if (SRC == SRC_PLAIN) {
-                    Elem<DT>::load8((const T *)a.x + src[i] * a.ldx + col, v[i]);
+                    Elem<DT>::unpack(r[i], v[i]);
                     if (a.row_scale) {
 #pragma unroll
                         for (int c = 0; c < 8; c++) v[i][c] *= sc[i];
