@@ -545,9 +545,20 @@ struct GroupedProblem {
                 pg[v] = *(const v4i *)pp;
                 pv[v] = *(const v4i *)(pp + H);
             }
+            // The four gate loads go out together and are converted afterwards.  (With the dtype test and
+            // the conversion inside the loop the compiler issued them one at a time, each behind a full
+            // wait for the one before: five memory latencies per slab of rows instead of two.)
+            if (p.gate_f32) {
 #pragma unroll
-            for (int v = 0; v < 4; v++)
-                gate[v] = p.gate_f32 ? ((const float *)p.gate)[pair[v]] : load_act<CDT>(p.gate, pair[v]);
+                for (int v = 0; v < 4; v++) gate[v] = ((const float *)p.gate)[pair[v]];
+            } else {
+                uint16_t raw[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) raw[v] = ((const uint16_t *)p.gate)[pair[v]];
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    gate[v] = CDT == MX_BF16 ? bits2f((uint32_t)raw[v] << 16) : (float)__builtin_bit_cast(_Float16, raw[v]);
+            }
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int m = row_of(t, L, i, v);
