@@ -46,6 +46,13 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
     return (uint32_t)v;
 }
 
+// 1 / (1 + e^-x) with the hardware exponential and reciprocal (v_exp_f32, v_rcp_f32: 1 ulp each).
+// Every SwiGLU in the library goes through this one function, so a fused epilogue and the
+// stand-alone quantizer of the same values agree bit for bit.  Written as a division the
+// compiler emitted the IEEE sequence (v_div_scale x2, v_rcp, four v_fma, v_div_fmas,
+// v_div_fixup): ten instructions per value, a sixth of the expert GEMM2-dgrad epilogue.
+__device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+
 // Element loaders: 8 consecutive elements starting at p (16-byte aligned for 16-bit types).
 template <int DT>
 struct Elem;

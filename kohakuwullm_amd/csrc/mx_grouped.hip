@@ -119,7 +119,7 @@ __device__ __forceinline__ void atomic_add2(void *base, int64_t off, float a, fl
     }
 }
 
-__device__ __forceinline__ float sigmoid_f(float x) { return __fdividef(1.0f, 1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return sigmoid_f32(x); }
 
 // Reductions over neighbouring lanes.  A lane owns 8 (GEMM1: 4) consecutive channels of a row
 // and its neighbours own the next ones, so a 32-channel MX block is a quad (GEMM1: 8 lanes)

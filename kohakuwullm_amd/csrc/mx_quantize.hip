@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256) void quant_dual_batch_kernel(QuantBatchArgs b)
     quant_tile<true>(v, b.o[j], M, K, m0, k0, tile, tscale);
 }
 
-__device__ __forceinline__ float sigmoid_fast(float x) { return __fdividef(1.0f, 1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoid_fast(float x) { return sigmoid_f32(x); }
 
 // h = silu(g) * u from the fused projection output gu (M, 2H) (gate half first), quantized
 // along both axes: (q,s) (M,H) for the down projection's forward, (qT,sT) (H,M) for its wgrad.
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows_kernel(const void *__re
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             float gv = a[u][i];
-            v[i] = gv * __fdividef(1.0f, 1.0f + __expf(-gv)) * b[u][i];
+            v[i] = gv * sigmoid_f32(gv) * b[u][i];
         }
         float amax = quad_max(amax8(v));
         uint32_t byte = scale_byte(amax);
