@@ -580,13 +580,13 @@ struct GroupedProblem {
                         const int word = hc[v][e >> 2];
                         const v2f pairv = (e & 2) ? __builtin_amdgcn_cvt_pk_f32_fp8(word, true)
                                                   : __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
-                        const float hval = pairv[e & 1] * hscale;
-                        dot += a[e] * hval;
-                        const float dh = a[e] * gate[v];
+                        dot += a[e] * pairv[e & 1];  // times the block's power-of-two scale once, below (exact)
                         const float sg = sigmoid_f(gq[e]);
-                        dg[e] = dh * vq[e] * sg * (1.0f + gq[e] * (1.0f - sg));
-                        dv[e] = dh * gq[e] * sg;
+                        const float dhs = a[e] * gate[v] * sg;
+                        dg[e] = dhs * vq[e] * (1.0f + gq[e] * (1.0f - sg));
+                        dv[e] = dhs * gq[e];
                     }
+                    dot *= hscale;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) dg[e] = dv[e] = 0.0f;
