@@ -1,4 +1,4 @@
-"""The benchmark configurations at their full sizes: attention projections, routed experts, outlier stress.
+"""The benchmark configurations at their full sizes: dense feed-forward, attention projections, routed experts, outlier stress.
 
 The CPU oracle cannot redo a whole 8192^3 product in seconds, so each case checks
   * quantizers bit for bit on the whole tensor (the C oracle quantizes 67M elements in about a second),
@@ -19,6 +19,7 @@ sys.path.insert(0, str(Path(__file__).resolve().parent.parent))
 
 import bench  # noqa: E402
 from conftest import SEED  # noqa: E402
+from mx_checks import assert_codes_equal_up_to_ties  # noqa: E402
 from test_gpu_moe import _expert_oracle  # noqa: E402
 
 pytestmark = pytest.mark.gpu
@@ -30,6 +31,108 @@ F8 = torch.float8_e4m3fn
 
 def _u8(t):
     return t.view(torch.uint8).cpu()
+
+
+# ----------------------------------------------------------------------------- dense SwiGLU feed-forward
+
+
+def test_dense_ffn_full_size(oracle):
+    """The benchmarked step (tokens 16384, dim 1536, ffn 4096) through ``mxfp8_swiglu_mlp``, on the benchmark's data.
+
+    The fused function is first shown equal, bit for bit, to its launches issued one by one (which exposes
+    the intermediates: the launch plan is the measured one, stage-major operands, the three backward products
+    in one batched launch).  Then every stage is held to the oracle on samples: quantizers on the whole
+    tensors, GEMM rows and columns against the fp64 dequantize-then-matmul on the operands the device used,
+    the SwiGLU casts against the oracle's evaluation up to rounding ties.
+    """
+    from kohakuwullm_amd.kernels.mxfp8.mlp import mxfp8_swiglu_mlp, swiglu_bwd_mx_dual, swiglu_mx_dual
+    from kohakuwullm_amd.kernels.mxfp8.quantize import (
+        mxfp8_matmul_pq, mxfp8_matmul_pq_batch, quantize_mx, quantize_mx_cols, quantize_mx_dual, rows_of_stage_major)
+
+    x, w_in, w_out, dy = bench.make_inputs(bench.TOKENS)
+    tokens, dim = x.shape
+    hid = w_out.shape[1]
+    xd, wi, wo = (t.to(DEV).requires_grad_(True) for t in (x, w_in, w_out))
+    dyd = dy.to(DEV)
+    packed = (quantize_mx(wi.detach()), quantize_mx_cols(wi.detach()), quantize_mx(wo.detach()), quantize_mx_cols(wo.detach()))
+    y = mxfp8_swiglu_mlp(xd, wi, wo, packed)
+    y.backward(dyd)
+    y, dx, dw_in, dw_out = y.detach(), xd.grad, wi.grad, wo.grad
+
+    # the same launches one by one
+    xq, xs, xtq, xts = quantize_mx_dual(xd.detach(), stage_major_t=True)
+    gu = mxfp8_matmul_pq(xq, xs, *packed[0])
+    hq, hs, htq, hts = swiglu_mx_dual(gu, stage_major_t=True)
+    assert torch.equal(mxfp8_matmul_pq(hq, hs, *packed[2]), y)
+    dq, ds, dtq, dts = quantize_mx_dual(dyd, stage_major_t=True)
+    dh = mxfp8_matmul_pq(dq, ds, *packed[3])
+    pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu, stage_major=True)
+    products = [(pq, ps, *packed[1]), (ptq, pts, xtq, xts), (dtq, dts, htq, hts)]
+    together = mxfp8_matmul_pq_batch(products)
+    for got, want in zip(together, (dx, dw_in, dw_out)):
+        assert torch.equal(got, want)
+    # the batched launch against each product launched alone: the same fp32 sums up to the order of their
+    # K pieces, then one bf16 rounding
+    for got, prob in zip(together, products):
+        alone = mxfp8_matmul_pq(*prob)
+        assert oracle.rel_error(got.cpu(), alone.double().cpu()) < 2e-3
+
+    # quantizers, whole tensors, bit for bit (stage-major codes read back as rows)
+    for t, (q, s, qt, st) in ((x, (xq, xs, xtq, xts)), (dy, (dq, ds, dtq, dts))):
+        rq, rs = oracle.quantize_rows(t)
+        cq, cs = oracle.quantize_cols(t)
+        assert torch.equal(_u8(q), rq) and torch.equal(s.cpu(), rs)
+        assert torch.equal(_u8(rows_of_stage_major(qt)), cq) and torch.equal(st.cpu(), cs)
+    win_f, win_d = oracle.quantize_rows(w_in), oracle.quantize_cols(w_in)
+    wout_f, wout_d = oracle.quantize_rows(w_out), oracle.quantize_cols(w_out)
+    for dev_pair, ref_pair in zip(packed, (win_f, win_d, wout_f, wout_d)):
+        assert torch.equal(_u8(dev_pair[0]), ref_pair[0]) and torch.equal(dev_pair[1].cpu(), ref_pair[1])
+
+    g = torch.Generator().manual_seed(SEED)
+    rows = torch.randperm(tokens, generator=g)[:192].sort().values
+    rd = rows.to(DEV)
+    # forward, sampled token rows
+    gu_rows = gu[rd].cpu()
+    assert oracle.rel_error(gu_rows, oracle.gemm_nt(_u8(xq[rd]), xs[rd].cpu(), *win_f)) < TOL
+    gate, up = gu_rows.float().chunk(2, dim=-1)
+    h_rows = gate * torch.sigmoid(gate) * up
+    ties = assert_codes_equal_up_to_ties(oracle, hq[rd], hs[rd], h_rows, what="h along H")
+    assert ties[0] < 5e-3 * h_rows.numel()
+    assert oracle.rel_error(y[rd].cpu(), oracle.gemm_nt(_u8(hq[rd]), hs[rd].cpu(), *wout_f)) < TOL
+    # backward, the same rows
+    dh_rows = dh[rd].cpu()
+    assert oracle.rel_error(dh_rows, oracle.gemm_nt(_u8(dq[rd]), ds[rd].cpu(), *wout_d)) < TOL
+    sg = torch.sigmoid(gate)
+    dpre_rows = torch.cat([dh_rows.float() * up * sg * (1 + gate * (1 - sg)), dh_rows.float() * gate * sg], dim=-1)
+    pq_rows = rows_of_stage_major(pq[:, rd])
+    terms = torch.cat([(dh_rows.float() * up * sg).abs() * (1 + gate.abs() * (1 - sg)), (dh_rows.float() * gate * sg).abs()], dim=-1)
+    ties = assert_codes_equal_up_to_ties(oracle, pq_rows, ps[rd], dpre_rows, ulps=8, what="dpre along 2H", magnitude=terms)
+    assert ties[0] < 5e-3 * dpre_rows.numel()
+    assert oracle.rel_error(dx[rd].cpu(), oracle.gemm_nt(_u8(pq_rows), ps[rd].cpu(), *win_d)) < TOL
+
+    # token-axis casts of h and dpre: four sampled panels of 128 tokens, every channel
+    for panel in torch.randperm(tokens // 128, generator=g)[:4].tolist():
+        tok = slice(panel * 128, panel * 128 + 128)
+        gate, up = gu[tok].cpu().float().chunk(2, dim=-1)
+        sg = torch.sigmoid(gate)
+        h_t = (gate * sg * up).t().contiguous()
+        assert_codes_equal_up_to_ties(oracle, htq[panel], hts[:, panel * 4 : panel * 4 + 4], h_t, what="h along tokens")
+        dh_p = dh[tok].cpu().float()
+        dpre_t = torch.cat([dh_p * up * sg * (1 + gate * (1 - sg)), dh_p * gate * sg], dim=-1).t().contiguous()
+        terms = torch.cat([(dh_p * up * sg).abs() * (1 + gate.abs() * (1 - sg)), (dh_p * gate * sg).abs()], dim=-1).t().contiguous()
+        assert_codes_equal_up_to_ties(oracle, ptq[panel], pts[:, panel * 4 : panel * 4 + 4], dpre_t, ulps=8, what="dpre along tokens",
+                                      magnitude=terms)
+
+    # weight gradients: sampled output rows against all input channels, and sampled input channels against
+    # all output rows, contracting all 16384 tokens on the device's own token-axis operands
+    xt_cpu, ht_cpu = (_u8(rows_of_stage_major(xtq)), xts.cpu()), (_u8(rows_of_stage_major(htq)), hts.cpu())
+    pt_cpu, dt_cpu = (_u8(rows_of_stage_major(ptq)), pts.cpu()), (_u8(rows_of_stage_major(dtq)), dts.cpu())
+    for dw, a, b in ((dw_in, pt_cpu, xt_cpu), (dw_out, dt_cpu, ht_cpu)):
+        pick = torch.randperm(a[0].shape[0], generator=g)[:48].sort().values
+        assert oracle.rel_error(dw[pick.to(DEV)].cpu(), oracle.gemm_nt(a[0][pick], a[1][pick], *b)) < TOL
+        pick = torch.randperm(b[0].shape[0], generator=g)[:32].sort().values
+        assert oracle.rel_error(dw[:, pick.to(DEV)].cpu(), oracle.gemm_nt(*a, b[0][pick], b[1][pick])) < TOL
+    assert hid * 2 == w_in.shape[0] and dw_in.shape == w_in.shape and dw_out.shape == w_out.shape
 
 
 # ----------------------------------------------------------------------------- attention projections

@@ -9,6 +9,8 @@ import torch
 
 from conftest import SEED
 
+from mx_checks import assert_codes_equal_up_to_ties  # noqa: E402
+
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
@@ -155,10 +157,12 @@ def test_swiglu_mx(oracle):
     q, s = swiglu_mx(g.to(DEV), u.to(DEV))
     qr, sr = oracle.swiglu_quantize_rows(g, u)
     q, s = q.view(torch.uint8).cpu(), s.cpu()
-    # the device sigmoid uses the hardware exp/rcp: an fp32 ulp can flip a rounding tie
-    assert (s != sr).float().mean() < 1e-3
-    assert (q != qr).float().mean() < 5e-3
     act = g.float() * torch.sigmoid(g.float()) * u.float()
+    # the device sigmoid uses the hardware exp/rcp: a value a few fp32 ulp away can fall on the other side of
+    # a rounding boundary.  Only such ties may differ, and few of them.
+    n_q, n_s = assert_codes_equal_up_to_ties(oracle, q, s, act, what="swiglu_mx")
+    assert n_s < 1e-3 * s.numel() and n_q < 5e-3 * q.numel()
+    assert (s != sr).sum() <= n_s + 1 and (q != qr).float().mean() < 5e-3  # the C oracle's libm agrees with torch's to the same ties
     assert oracle.rel_error(oracle.dequant(q, s), act) < 0.04
     # chunked halves of one projection, as GLUMLP produces them
     both = torch.cat([g, u], dim=1).to(DEV)
