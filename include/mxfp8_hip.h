@@ -6,13 +6,15 @@
  *     launches on the stream the caller passes (a hipStream_t travelling as
  *     void*; NULL = the default stream);
  *   - returns MX_OK or a negative MX_E* code and never throws;
- *   - allocates nothing, with one exception: the first mx_gemm_nt on a given
- *     (device, stream) whose shape leaves the last round of tiles mostly empty
- *     allocates a scratch of 2 x 256 KiB per CU (128 MiB on MI355X) that is kept
- *     for the life of the process; the call skips that optimisation instead
- *     when the stream is being captured or the allocation fails;
- *   - is thread-safe; calls that share a stream share that scratch, which is
- *     safe because work on one stream runs in order.
+ *   - allocates nothing: outputs, index scratch and the GEMMs' K-split workspace
+ *     all come from the caller (mx_gemm_workspace_bytes, mx_expert_sort_workspace);
+ *   - is re-entrant and thread-safe: no state is kept between calls besides two
+ *     write-once caches (the CU count per device ordinal, and "the large-LDS
+ *     attribute of this kernel is set" per kernel and device);
+ *   - refuses with MX_ECAPTURE, before launching anything, when the stream is
+ *     being captured into a HIP graph: recording this library's launches ended a
+ *     process inside graph instantiation and stays switched off until the cause
+ *     is known.
  *
  * The reference (KohakUwULLM) has no FFI; each function cites the reference
  * Python/Triton interface it stands in for (paths relative to the reference tree).
@@ -30,14 +32,15 @@
 extern "C" {
 #endif
 
-#define MX_ABI_VERSION 1
+#define MX_ABI_VERSION 2
 
 enum mx_status {
     MX_OK = 0,
     MX_EINVAL = -1,      /* a size/stride/alignment contract is violated (ValueError upstream) */
     MX_EUNSUPPORTED = -2, /* well-formed request this build has no kernel for */
     MX_ELAUNCH = -3,     /* the HIP runtime refused the launch */
-    MX_ENODEV = -4       /* the current device is not gfx950 */
+    MX_ENODEV = -4,      /* the current device is not gfx950 */
+    MX_ECAPTURE = -5     /* the stream is being captured into a graph: nothing was launched */
 };
 
 enum mx_dtype { MX_BF16 = 0, MX_FP16 = 1, MX_FP32 = 2 };
@@ -207,14 +210,30 @@ int mx_unswizzle_scales(const uint8_t *swizzled, int64_t rows, int64_t cols, uin
  * One entry serves forward (X W^T), dgrad (dY (W^T)^T) and wgrad (dY^T (X^T)^T)
  * because the quantizers deliver every operand K-minor.  lda == 128 (ldb == 128) with
  * K > 128 reads A (B) in the stage-major layout described at mx_quantize_dual (K % 128 == 0).
+ * workspace: device scratch of workspace_bytes bytes (16-byte aligned) or NULL.  With at least
+ * mx_gemm_workspace_bytes() of it, a shape whose last round of tiles leaves most of the GPU idle
+ * has the K stages of those tiles dealt over all workgroups (fp32 partial tiles go through the
+ * workspace, a second kernel adds them in a fixed order).  With less, every tile is computed
+ * whole: same product, fp32 sums in another order, slower on such shapes.  The workspace holds
+ * nothing between calls; calls that may overlap in time need separate ones.
  * Replaces mxfp8_matmul_pq / _mxfp8_matmul_pq
  * (src/kohakuwullm/kernels/mxfp8/quantize.py:242-371) and the cuBLAS route
- * mxfp8_mm_swizzled (src/kohakuwullm/kernels/mxfp8/interop.py:51-122).
+ * mxfp8_mm_swizzled (src/kohakuwullm/kernels/mxfp8/interop.py:51-122); the reference's
+ * wrapper allocates what its kernel writes through torch (quantize.py:328-371), which is what
+ * the workspace argument leaves to this library's caller.
  */
 int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs,
                void *c, int c_dtype, int64_t M, int64_t N, int64_t K,
                int64_t lda, int64_t ldas, int64_t ldb, int64_t ldbs, int64_t ldc,
-               int epilogue, void *stream);
+               int epilogue, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * Bytes of workspace that let mx_gemm_nt, mx_gemm_nt_batch and mx_grouped_wgrad_nt split K on the
+ * current device: two fp32 tiles of 256 x 256 per compute unit (128 MiB on MI355X).  It depends
+ * on the device only, never on a shape (the reference's rule for launch plans: a pure function of
+ * static properties, never of the token count, src/kohakuwullm/kernels/mxfp8/quantize.py:59-62).
+ */
+int64_t mx_gemm_workspace_bytes(void);
 
 /*
  * Up to any number of independent products C_j = deq(A_j) deq(B_j)^T behind as few
@@ -223,7 +242,8 @@ int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const ui
  * fill the GPU one by one: DGRAD with WGRAD of a linear layer, the three products that
  * end a SwiGLU block's backward.  All outputs have dtype c_dtype.  `problems` is a
  * HOST array, read before the call returns.  Results are those of `count` calls of
- * mx_gemm_nt with MX_EPI_NONE.
+ * mx_gemm_nt with MX_EPI_NONE.  workspace as in mx_gemm_nt (one for the whole call); without it
+ * products are not cut into K slices and a sparse last round is not split.
  * Replaces the back-to-back launches of the reference's backward
  * (src/kohakuwullm/kernels/mxfp8/linear.py:66-74: dx then dw; models/components/mlp.py:68-73
  * under autograd).
@@ -233,7 +253,8 @@ typedef struct mx_gemm_problem {
     void *c;
     int64_t M, N, K, lda, ldas, ldb, ldbs, ldc;
 } mx_gemm_problem;
-int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *stream);
+int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *workspace,
+                     int64_t workspace_bytes, void *stream);
 
 /*
  * ---- routed experts -------------------------------------------------------------------
@@ -314,7 +335,8 @@ int mx_experts_combine(const void *y, int64_t ldy, const int32_t *order, const i
  * dpre quantized along the tokens in the padded layout of mx_quantize_cols_grouped, bit for
  * bit what that quantizer makes of dpre; dpre itself may then be NULL and is not written.
  * Replaces _experts_gemm2_dgrad (src/kohakuwullm/kernels/mxfp8/experts_bwd.py:29-164); with
- * ptq it also stands in for the dpre pass of _quantize_cols_grouped (quant.py, WGRAD of GEMM1).
+ * ptq it also stands in for the pass over the stored dpre that feeds GEMM1's WGRAD
+ * (_launch_wgrad(dpre, x, ...), src/kohakuwullm/kernels/mxfp8/moe.py:311-324).
  */
 int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int64_t T, int64_t lddq, int64_t ldds,
                            const int32_t *token_of, const int32_t *order, const void *gate, int gate_dtype,
@@ -349,11 +371,13 @@ int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, int64_t C, i
  * multiply in 16 bits.
  * When both scale pitches leave 12 readable bytes behind a row's last stage (ldas, ldbs >=
  * mpad/32 + 12) the kernel fetches a row's scale bytes 16 at a time instead of 4.
+ * workspace as in mx_gemm_nt: with mx_gemm_workspace_bytes() of it the K stages of the experts that
+ * have rows are dealt evenly over the workgroups when their tiles alone would leave CUs idle.
  */
 int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t lda, int64_t ldas, const uint8_t *bq,
                         const uint8_t *bs, int64_t ldb, int64_t ldbs, const int32_t *offsets, int64_t E,
                         int64_t M, void *dw, int dw_dtype, int64_t stride_dwe, int64_t lddw, int64_t N,
-                        int64_t Kout, void *stream);
+                        int64_t Kout, void *workspace, int64_t workspace_bytes, void *stream);
 
 /* ---- expert dispatch either side of the routed-expert GEMMs ------------------------------ */
 
@@ -420,6 +444,29 @@ int mx_combine_routed_backward(const void *grad_out, int64_t ldg, const void *ro
                                const int32_t *valid_rows, int64_t n, int64_t d, int64_t num_tokens, int64_t pairs,
                                void *grad_rows, int64_t ldgr, float *grad_weight, void *stream);
 
+/* ---- measured denominators ---------------------------------------------------------------- */
+
+/*
+ * One streaming pass over device buffers, for the bandwidth the quantizers are priced against:
+ *   kind 0  read:  reads out_bytes of a (c receives 4 bytes per launched thread, at most 16 MiB);
+ *   kind 1  copy:  c = a, out_bytes each way;
+ *   kind 2  triad: c = a + 2 b on fp32, out_bytes per operand;
+ *   kind 3  2:1:   reads 2 * out_bytes of a, writes out_bytes of c (a 16-bit -> 8-bit cast's traffic).
+ * out_bytes % 16 == 0, 16-byte aligned pointers.  The reference measures the same trio on its device
+ * and takes the best as its denominator (src/kohakuwullm/bench/core/timing.py:231-268).
+ */
+int mx_ubench_stream(int kind, const void *a, const void *b, void *c, int64_t out_bytes, void *stream);
+
+/*
+ * Register-resident loop of the block-scaled fp8 MFMA (wide == 0: v_mfma_scale_f32_16x16x128_f8f6f4 with
+ * 8 independent accumulator tiles per wave, wide != 0: ..._32x32x64_... with 4), 8 waves on every CU,
+ * `iters` rounds; operands zero or (random != 0) a per-lane hash.  Returns the number of MFMA
+ * instructions the launch issues (each 2 * 16*16*128 = 65536 or 2 * 32*32*64 = 131072 FLOP) or a
+ * negative mx_status.  out: one float per launched thread (512 x CUs).  The reference's rule for a
+ * compute ceiling: measured from registers with independent accumulators
+ * (docs/internals/kernel-convention.md:14-33).
+ */
+int64_t mx_ubench_mfma(int wide, int iters, int random, float *out, int64_t out_floats, void *stream);
 
 #ifdef __cplusplus
 }

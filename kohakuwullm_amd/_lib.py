@@ -17,7 +17,8 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmxfp8_hip.so")
 
-MX_OK, MX_EINVAL, MX_EUNSUPPORTED, MX_ELAUNCH, MX_ENODEV = 0, -1, -2, -3, -4
+MX_OK, MX_EINVAL, MX_EUNSUPPORTED, MX_ELAUNCH, MX_ENODEV, MX_ECAPTURE = 0, -1, -2, -3, -4, -5
+MX_ABI_VERSION = 2
 MX_DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
 _i64, _p, _ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
@@ -51,7 +52,7 @@ SIGNATURES = {
     "mx_quantize_cols_grouped": (
         _ci, [_p, _ci, _i64, _i64, _ci, _p, _p, _ci, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _p]),
     "mx_grouped_wgrad_nt": (
-        _ci, [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p]),
+        _ci, [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p]),
     "mx_rmsnorm_quantize": (
         _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, ctypes.c_float, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
     "mx_rmsnorm_backward": (
@@ -64,8 +65,11 @@ SIGNATURES = {
         _ci, [_p, _i64, _p, _i64, _ci, _p, _ci, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _p]),
     "mx_swizzle_scales": (_ci, [_p, _i64, _i64, _i64, _p, _p]),
     "mx_unswizzle_scales": (_ci, [_p, _i64, _i64, _p, _i64, _p]),
-    "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p]),
-    "mx_gemm_nt_batch": (_ci, [_p, _ci, _ci, _p]),
+    "mx_gemm_nt": (_ci, [_p, _p, _p, _p, _p, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _p, _i64, _p]),
+    "mx_gemm_workspace_bytes": (_i64, []),
+    "mx_gemm_nt_batch": (_ci, [_p, _ci, _ci, _p, _i64, _p]),
+    "mx_ubench_stream": (_ci, [_ci, _p, _p, _p, _i64, _p]),
+    "mx_ubench_mfma": (_i64, [_ci, _ci, _ci, _p, _i64, _p]),
 }
 
 
@@ -118,12 +122,32 @@ def check(status: int, what: str) -> None:
     msg = load().mx_strerror(status).decode()
     if status == MX_EINVAL:
         raise ValueError(f"{what}: {msg}")
+    if status == MX_ECAPTURE:
+        raise MXFP8LibraryError(
+            f"{what}: {msg}.  Keep MXFP8 layers out of torch.cuda.graph / hipStreamBeginCapture regions."
+        )
     raise MXFP8LibraryError(f"{what}: {msg} (status {status})")
 
 
 def stream_of(t: torch.Tensor) -> int:
     """The raw hipStream_t PyTorch is currently issuing on for ``t``'s device."""
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_WORKSPACE_BYTES: dict[int, int] = {}
+
+
+def gemm_workspace(t: torch.Tensor) -> torch.Tensor:
+    """Scratch for the K splits of ``mx_gemm_nt`` / ``mx_gemm_nt_batch`` / ``mx_grouped_wgrad_nt`` on ``t``'s device.
+
+    It comes from PyTorch's caching allocator on the current stream, per call: the block is reused by the
+    next call on that stream and is never touched by work on another one.  The library itself allocates nothing.
+    """
+    index = t.device.index if t.device.index is not None else torch.cuda.current_device()
+    if index not in _WORKSPACE_BYTES:
+        with torch.cuda.device(index):
+            _WORKSPACE_BYTES[index] = int(load().mx_gemm_workspace_bytes())
+    return torch.empty(_WORKSPACE_BYTES[index], dtype=torch.uint8, device=t.device)
 
 
 def require_gpu(t: torch.Tensor, name: str) -> None:

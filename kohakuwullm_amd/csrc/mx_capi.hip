@@ -12,6 +12,8 @@ extern "C" const char *mx_strerror(int status) {
     case MX_EUNSUPPORTED: return "unsupported: no kernel in this build covers the request";
     case MX_ELAUNCH: return "the HIP runtime refused the kernel launch";
     case MX_ENODEV: return "the device is not a gfx950 (MI355X-class) GPU";
+    case MX_ECAPTURE:
+        return "the stream is being captured into a graph: this library refuses to be recorded (run it eagerly)";
     default: return "unknown status";
     }
 }

@@ -10,6 +10,10 @@
 
 namespace mx {
 
+// Whether work on `st` is being recorded into a graph (mx_gemm.hip).  Every entry point asks before it
+// launches and returns MX_ECAPTURE: recording this library's launches is switched off.
+bool stream_is_capturing(hipStream_t st);
+
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));

@@ -393,6 +393,7 @@ extern "C" int mx_expert_counts(const void *flat_idx, int idx_bytes, int64_t n, 
         return MX_EINVAL;
     if (num_buckets > MAX_COUNT_BUCKETS) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     dispatch_fill_kernel<<<dim3((unsigned)((num_buckets + 255) / 256)), dim3(256), 0, st>>>(counts, num_buckets, 0);
     if (n) {
         const int64_t per_block = 1024;
@@ -423,6 +424,7 @@ extern "C" int mx_expert_sort(const void *flat_expert, int idx_bytes, int64_t n,
     const int64_t need = mx_expert_sort_workspace(n, num_buckets);
     if (!workspace || workspace_len < need) return MX_EINVAL;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     const int rounds = sort_rounds(n), buckets = (int)num_buckets;
     const int chunks = (int)(need / num_buckets);
     const size_t lds = (size_t)buckets * sizeof(int32_t);
@@ -450,6 +452,7 @@ extern "C" int mx_combine_routed(const void *rows, int dtype, int64_t ld, const 
     const int64_t blocks = (num_tokens * (d / 8) + 255) / 256;
     if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     dispatch_fill_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>(inv, pairs, -1);
     if (n) combine_invert_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(order, valid_rows, n, pairs, inv);
     if (n && top_k > 1) combine_sort_kernel<<<dim3((unsigned)((num_tokens + 255) / 256)), dim3(256), 0, st>>>(inv, (int)top_k, num_tokens);
@@ -476,6 +479,7 @@ extern "C" int mx_combine_routed_backward(const void *grad_out, int64_t ldg, con
         (ld * esz) % 16 || (ldgr * esz) % 16)
         return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     if (pairs) dispatch_fill_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>((int32_t *)grad_weight, pairs, 0);
     if (n == 0 || d == 0) return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
     switch (dtype) {

@@ -3,10 +3,7 @@
 // Semantics: mxfp8_matmul_pq of the reference (src/kohakuwullm/kernels/mxfp8/quantize.py:242-371).
 // The kernel body lives in mx_gemm_core.h; this file supplies the dense problem policy,
 // the slow generic kernel for shapes the tiled kernel does not take, and the C entry point.
-#include <cstdlib>
-#include <map>
-#include <mutex>
-#include <utility>
+#include <atomic>
 
 #include "mx_gemm_core.h"
 
@@ -338,62 +335,53 @@ using namespace mx;
 static inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
 namespace mx {
+// CUs of the current device, asked of the runtime once per device ordinal.  The cache is a word per
+// ordinal written with the one value it can ever hold: no lock, no table that grows.
 int num_cus() {
-    static std::mutex lock;
-    static int cached[64];  // by device ordinal; 0 = not asked yet
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    std::lock_guard<std::mutex> guard(lock);
-    if (!cached[dev]) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+bool allow_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    const uint64_t bit = 1ull << dev;
+    if (done.load(std::memory_order_acquire) & bit) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
     }
-    return cached[dev];
+    done.fetch_or(bit, std::memory_order_release);
+    return true;
 }
 
-bool allow_dynamic_lds(const void *kernel, int bytes) {
-    static std::mutex lock;
-    static std::map<std::pair<int, const void *>, bool> done;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return false;
-    std::lock_guard<std::mutex> guard(lock);
-    auto key = std::make_pair(dev, kernel);
-    auto it = done.find(key);
-    if (it != done.end()) return it->second;
-    const bool ok = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
-    if (!ok) (void)hipGetLastError();
-    done[key] = ok;
-    return ok;
-}
-}  // namespace mx
-
-// Scratch of the K splits (dense and expert WGRAD): two fp32 tile slots per workgroup, kept per
-// (device, stream) for the life of the process so launches on different streams never share it.
-namespace mx {
-float *split_scratch(hipStream_t st, int cus, size_t tile_floats) {
-    static std::mutex lock;
-    static std::map<std::pair<int, hipStream_t>, float *> table;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-    std::lock_guard<std::mutex> guard(lock);
-    auto key = std::make_pair(dev, st);
-    auto it = table.find(key);
-    if (it != table.end()) return it->second;
+bool stream_is_capturing(hipStream_t st) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    const hipError_t e = hipStreamIsCapturing(st, &cap);
+    if (e != hipSuccess) {
         (void)hipGetLastError();
-        return nullptr;  // no allocation while the stream is being captured: whole tiles only, this time
+        // the capture family of errors (e.g. the legacy stream while another stream captures in global
+        // mode) counts as capturing; anything else (no device) is left for the launch itself to report
+        return e >= hipErrorStreamCaptureUnsupported && e <= hipErrorStreamCaptureWrongThread;
     }
-    float *slots = nullptr;
-    if (hipMalloc((void **)&slots, (size_t)cus * 2 * tile_floats * sizeof(float)) != hipSuccess) {
-        (void)hipGetLastError();
-        slots = nullptr;
-    }
-    table[key] = slots;  // a failed allocation is remembered: the library keeps working on whole tiles
-    return slots;
+    return cap != hipStreamCaptureStatusNone;
 }
 }  // namespace mx
+
+// fp32 tile slots a caller's workspace holds for the K splits (dense and expert WGRAD): the kernels use at
+// most two per workgroup, so 2 x CUs slots of one 256 x 256 tile are all they can ever take.
+static inline int64_t slot_bytes() { return (int64_t)256 * 256 * sizeof(float); }
+static inline int workspace_slots(const void *ws, int64_t bytes) {
+    if (!ws || bytes <= 0 || ((uintptr_t)ws & 15)) return 0;
+    const int64_t n = bytes / slot_bytes();
+    return n > 0x7FFFFFFF ? 0x7FFFFFFF : (int)n;
+}
 
 // Which scale fetch (SCALES_*) a problem's K and scale pointers allow.
 static int scale_mode(const DenseArgs &a) {
@@ -402,17 +390,8 @@ static int scale_mode(const DenseArgs &a) {
     return SCALES_BYTES;
 }
 
-// MX_GEMM_SPLIT=0 in the environment keeps every tile whole (for A/B timing and debugging).
-static bool split_mode() {
-    static const bool on = [] {
-        const char *e = std::getenv("MX_GEMM_SPLIT");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
 template <typename S, int CDT>
-static int launch_tiled(DenseArgs a, hipStream_t st) {
+static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st) {
     a.tiles_m = (a.M + S::BM - 1) / S::BM;
     a.tiles_n = (a.N + S::BN - 1) / S::BN;
     const int esz = CDT == MX_FP32 ? 4 : 2;
@@ -429,13 +408,13 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
     // tile, so no tile is cut into more than 9 pieces.
     const int rest = (int)(work % cus);
     const int KT = ((a.K + 127) >> 7), KT4 = (KT + 3) & ~3;
-    if (split_mode() && a.split_k == 1 && !a.accumulate && rest > 0 && KT4 >= 8) {
+    if (a.split_k == 1 && !a.accumulate && rest > 0 && KT4 >= 8) {
         int64_t q = ((int64_t)rest * KT4 + cus - 1) / cus;
         if (q < KT4 / 8) q = KT4 / 8;
         q = (q + 3) & ~(int64_t)3;
         const double pieces = (double)rest * KT4 / q + rest;
         const double gain = (double)(KT4 - q), cost = 4.0 + 0.15 * pieces;
-        float *slots = gain > 1.25 * cost ? split_scratch(st, cus, (size_t)S::BM * S::BN) : nullptr;
+        float *slots = gain > 1.25 * cost && ws_slots >= 2 * cus ? ws : nullptr;  // two slots per workgroup
         if (slots) {
             a.sk_tiles = rest;
             a.dp_tiles = (int)work - rest;
@@ -444,11 +423,10 @@ static int launch_tiled(DenseArgs a, hipStream_t st) {
         }
     }
     dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
-    auto kern = mode == SCALES_VEC16   ? gemm_nt_kernel<S, CDT, SCALES_VEC16>
-                : mode == SCALES_DWORD ? gemm_nt_kernel<S, CDT, SCALES_DWORD>
-                                       : gemm_nt_kernel<S, CDT, SCALES_BYTES>;
-    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
-    kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    const int rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+                   : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
+                                          : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
+    if (rc != MX_OK) return rc;
     if (a.sk_tiles)
         split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * S::MT)), block, 0, st>>>(a);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
@@ -465,7 +443,7 @@ static bool tiled_ok(const DenseArgs &a) {
 }
 
 template <int CDT>
-static int gemm_dispatch(DenseArgs a, hipStream_t st) {
+static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st) {
     const int64_t M = a.M, N = a.N;
     if (!tiled_ok(a)) {
         if (a.accumulate || a.a_ks || a.b_ks) return MX_EUNSUPPORTED;  // the element-wise kernel reads row-major only
@@ -475,7 +453,7 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
                                                                                   a.lda, a.ldas, a.ldb, a.ldbs, a.ldc);
         return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
     }
-    return launch_tiled<DenseShape, CDT>(a, st);
+    return launch_tiled<DenseShape, CDT>(a, ws, ws_slots, st);
 }
 
 // Several products behind one launch, the eight XCDs shared out among them whole.  Every problem
@@ -487,10 +465,10 @@ static int gemm_dispatch(DenseArgs a, hipStream_t st) {
 // everyone's time) and the cheapest plan wins, against running the products one after the other
 // as well.
 template <int CDT>
-static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
+static int batch_dispatch(DenseArgs *probs, int count, float *ws, int ws_slots, hipStream_t st) {
     typedef DenseShape S;
     const int cus = num_cus();
-    bool fuse = count > 1 && count <= MX_BATCH_MAX && split_mode();
+    bool fuse = count > 1 && count <= MX_BATCH_MAX;
     DenseBatchArgs b;
     int64_t tiles[MX_BATCH_MAX], alone = 0;
     int KT[MX_BATCH_MAX];
@@ -516,7 +494,7 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
             int64_t q = (rest * KT4 + cus - 1) / cus;
             q = ((q < KT4 / 8 ? KT4 / 8 : q) + 3) & ~(int64_t)3;
             const double pieces = (double)rest * KT4 / q + rest, cost = 4.0 + 0.15 * pieces;
-            alone += KT4 >= 8 && (double)(KT4 - q) > 1.25 * cost ? q + (int64_t)cost : KT[j] + 4;
+            alone += KT4 >= 8 && ws_slots >= 2 * cus && (double)(KT4 - q) > 1.25 * cost ? q + (int64_t)cost : KT[j] + 4;
         }
         // A product with several full rounds of tiles runs well on its own (each XCD's 32 CUs
         // share A/B panels in L2, the ragged last round is K-split); confined to a part of the
@@ -533,7 +511,7 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     fuse = fuse && cus % 8 == 0 && count <= 8;
     if (fuse) {
         const int per_xcd = cus / 8;
-        const int slots = 2 * cus;  // fp32 tile slots of the scratch
+        const int slots = ws_slots < 2 * cus ? ws_slots : 2 * cus;  // fp32 tile slots the caller's workspace offers
         auto per_slice = [&](int j) { return (((KT[j] + slices[j] - 1) / slices[j]) + 3) & ~3; };
         auto units = [&](int j) { return tiles[j] * slices[j]; };
         auto finish = [&](int j) {
@@ -574,14 +552,11 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
     if (fuse) {
         bool any = false;
         for (int j = 0; j < count; j++) any = any || best_slices[j] > 1;
-        if (any) {
-            scratch = split_scratch(st, cus, (size_t)S::BM * S::BN);
-            if (!scratch) fuse = false;  // no scratch (allocation failed or the stream is being captured)
-        }
+        if (any) scratch = ws;  // the plan fitted its partial tiles into the workspace's slots
     }
     if (!fuse) {
         for (int j = 0; j < count; j++) {
-            int rc = gemm_dispatch<CDT>(probs[j], st);
+            int rc = gemm_dispatch<CDT>(probs[j], ws, ws_slots, st);
             if (rc != MX_OK) return rc;
         }
         return MX_OK;
@@ -600,11 +575,12 @@ static int batch_dispatch(DenseArgs *probs, int count, hipStream_t st) {
         b.prob[j] = a;
     }
     b.count = count;
-    auto kern = mode == SCALES_VEC16   ? gemm_nt_batch_kernel<S, CDT, SCALES_VEC16>
-                : mode == SCALES_DWORD ? gemm_nt_batch_kernel<S, CDT, SCALES_DWORD>
-                                       : gemm_nt_batch_kernel<S, CDT, SCALES_BYTES>;
-    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
-    kern<<<dim3((unsigned)cus), dim3(S::NTHR), S::LDS_BYTES, st>>>(b);
+    const dim3 grid((unsigned)cus), block(S::NTHR);
+    const int rc = mode == SCALES_VEC16 ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, b)
+                   : mode == SCALES_DWORD
+                       ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, b)
+                       : launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, b);
+    if (rc != MX_OK) return rc;
     for (int j = 0; j < count; j++)
         if (probs[j].split_k > 1)
             slice_reduce_kernel<S, CDT><<<dim3((unsigned)(tiles[j] * S::MT)), dim3(S::NTHR), 0, st>>>(probs[j]);
@@ -648,19 +624,24 @@ static int zero_matrix(void *c, int c_dtype, int64_t M, int64_t N, int64_t ldc, 
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
-extern "C" int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *stream) {
-    if (count < 0 || (count > 0 && !problems)) return MX_EINVAL;
+extern "C" int64_t mx_gemm_workspace_bytes(void) { return 2 * (int64_t)num_cus() * slot_bytes(); }
+
+extern "C" int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int c_dtype, void *workspace,
+                                int64_t workspace_bytes, void *stream) {
+    if (count < 0 || (count > 0 && !problems) || workspace_bytes < 0) return MX_EINVAL;
     if (c_dtype != MX_BF16 && c_dtype != MX_FP16 && c_dtype != MX_FP32) return MX_EINVAL;
     hipStream_t st = (hipStream_t)stream;
+    float *const ws = (float *)workspace;
+    const int ws_slots = workspace_slots(workspace, workspace_bytes);
     DenseArgs live[MX_BATCH_MAX];
     int n = 0;
     auto flush = [&]() -> int {
         int rc = MX_OK;
         if (n) {
             switch (c_dtype) {
-            case MX_BF16: rc = batch_dispatch<MX_BF16>(live, n, st); break;
-            case MX_FP16: rc = batch_dispatch<MX_FP16>(live, n, st); break;
-            default: rc = batch_dispatch<MX_FP32>(live, n, st); break;
+            case MX_BF16: rc = batch_dispatch<MX_BF16>(live, n, ws, ws_slots, st); break;
+            case MX_FP16: rc = batch_dispatch<MX_FP16>(live, n, ws, ws_slots, st); break;
+            default: rc = batch_dispatch<MX_FP32>(live, n, ws, ws_slots, st); break;
             }
         }
         n = 0;
@@ -672,6 +653,7 @@ extern "C" int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int 
         int rc = fill_args(probe, q.aq, q.a_scale, q.bq, q.b_scale, q.c, q.M, q.N, q.K, q.lda, q.ldas, q.ldb, q.ldbs, q.ldc);
         if (rc != MX_OK) return rc;
     }
+    if (count && stream_is_capturing(st)) return MX_ECAPTURE;
     for (int j = 0; j < count; j++) {
         const mx_gemm_problem &q = problems[j];
         if (q.M == 0 || q.N == 0) continue;
@@ -691,7 +673,9 @@ extern "C" int mx_gemm_nt_batch(const mx_gemm_problem *problems, int count, int 
 
 extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *bq, const uint8_t *bs, void *c,
                           int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldas, int64_t ldb,
-                          int64_t ldbs, int64_t ldc, int epilogue, void *stream) {
+                          int64_t ldbs, int64_t ldc, int epilogue, void *workspace, int64_t workspace_bytes,
+                          void *stream) {
+    if (workspace_bytes < 0) return MX_EINVAL;
     DenseArgs a;
     int rc = fill_args(a, aq, as, bq, bs, c, M, N, K, lda, ldas, ldb, ldbs, ldc);
     if (rc != MX_OK) return rc;
@@ -703,13 +687,16 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     if (c_dtype != MX_BF16 && c_dtype != MX_FP16 && c_dtype != MX_FP32) return MX_EINVAL;
     if (M == 0 || N == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (stream_is_capturing(st)) return MX_ECAPTURE;
+    float *const ws = (float *)workspace;
+    const int ws_slots = workspace_slots(workspace, workspace_bytes);
     if (K == 0)  // an empty contraction is a zero matrix
         return epi == MX_EPI_ACCUMULATE ? MX_OK : zero_matrix(c, c_dtype, M, N, ldc, st);
     a.accumulate = epi == MX_EPI_ACCUMULATE;
     a.split_k = split_k > 1 ? split_k : 1;
     switch (c_dtype) {
-    case MX_BF16: return gemm_dispatch<MX_BF16>(a, st);
-    case MX_FP16: return gemm_dispatch<MX_FP16>(a, st);
-    default: return gemm_dispatch<MX_FP32>(a, st);
+    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st);
+    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st);
+    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st);
     }
 }

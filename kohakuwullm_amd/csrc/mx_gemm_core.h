@@ -33,6 +33,8 @@
 //     buffers, the read of sub-tile j+1 in flight under the MFMAs of sub-tile j.
 #pragma once
 
+#include <atomic>
+
 #include "mx_common.h"
 
 namespace mx {
@@ -532,10 +534,19 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int &t
 }
 
 // Host-side launch helpers shared by the GEMM translation units (defined in mx_gemm.hip).
-// Both cache their answer: the per-launch path makes no HIP call besides the launch itself, which
-// is what a stream being captured into a graph tolerates (attribute calls from autograd's worker
-// thread count as unsafe during a capture and would invalidate it).
-int num_cus();                                   // CUs of the current device
-bool allow_dynamic_lds(const void *kernel, int bytes);  // hipFuncSetAttribute, once per kernel
+int num_cus();                            // CUs of the current device (cached per device ordinal)
+bool stream_is_capturing(hipStream_t st);  // true also when the capture status cannot be read
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per device; `done` has one bit per device ordinal.
+bool allow_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done);
+
+// Launch of a kernel that needs more than 64 KiB of dynamic LDS.  The "attribute already set" word is a
+// function-local static of this instantiation, i.e. one per kernel: no table shared between kernels, no lock.
+template <auto Kern, typename Args>
+int launch_with_lds(dim3 grid, dim3 block, int lds_bytes, hipStream_t st, const Args &a) {
+    static std::atomic<uint64_t> done{0};
+    if (!allow_dynamic_lds((const void *)Kern, lds_bytes, done)) return MX_ELAUNCH;
+    Kern<<<grid, block, lds_bytes, st>>>(a);
+    return MX_OK;
+}
 
 }  // namespace mx

@@ -21,7 +21,6 @@
 
 namespace mx {
 
-float *split_scratch(hipStream_t st, int cus, size_t tile_floats);  // mx_gemm.hip
 
 enum { MODE_PLAIN = 0, MODE_GEMM1 = 1, MODE_SCATTER = 2, MODE_DGRAD2 = 3 };
 
@@ -1161,9 +1160,9 @@ static int launch_grouped(GroupedArgs a, hipStream_t st) {
                       a.ldws % 16 == 0 && a.stride_wse % 16 == 0;
     const int cus = num_cus();
     dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
-    auto kern = k512 ? grouped_kernel<S, MODE, CDT, SCALES_VEC16> : grouped_kernel<S, MODE, CDT, SCALES_DWORD>;
-    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
-    kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    const int rc = k512 ? launch_with_lds<grouped_kernel<S, MODE, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+                        : launch_with_lds<grouped_kernel<S, MODE, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
+    if (rc != MX_OK) return rc;
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
@@ -1198,6 +1197,7 @@ extern "C" int mx_grouped_gemm_nt(const uint8_t *xq, const uint8_t *xs, int64_t 
     if (!sizes_ok(E, M, N, K) || ldx < K || ldw < K || ldo < N) return MX_EINVAL;
     if (M == 0 || N == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     GroupedArgs a = base_args(xq, xs, ldx, ldxs, index, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, N, K);
     a.out = out, a.ldo = ldo;
     const int esz = out_dtype == MX_FP32 ? 4 : 2;
@@ -1240,6 +1240,7 @@ extern "C" int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T,
     if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 8) || ldpre % 4)) ||
         (htq && (!aligned(htq, 16) || ldhtq % 16 || !aligned(hts, 4) || ldhts % 4)))
         return MX_EUNSUPPORTED;
+    if (mx::stream_is_capturing((hipStream_t)stream)) return MX_ECAPTURE;
     return launch_grouped_dt<MODE_GEMM1>(act_dtype, a, (hipStream_t)stream);
 }
 
@@ -1256,6 +1257,7 @@ extern "C" int mx_experts_scatter_gemm(const uint8_t *aq, const uint8_t *as, int
     a.token_of = token_of, a.order = order, a.gate = gate, a.gate_f32 = gate_dtype == MX_FP32;
     a.out = out, a.ldo = ldo;
     if (K == 0 || !tiled_ok(a, a_rows) || !aligned(out, 4) || ldo % 2) return MX_EUNSUPPORTED;
+    if (mx::stream_is_capturing((hipStream_t)stream)) return MX_ECAPTURE;
     return launch_grouped_dt<MODE_SCATTER>(out_dtype, a, (hipStream_t)stream);
 }
 
@@ -1285,6 +1287,7 @@ extern "C" int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int6
         ldpre % 8 || H % 8 || !aligned(dpq, 8) || lddpq % 8 ||
         (ptq && (!aligned(ptq, 16) || ldptq % 16 || !aligned(pts, 4) || ldpts % 4)))
         return MX_EUNSUPPORTED;
+    if (mx::stream_is_capturing((hipStream_t)stream)) return MX_ECAPTURE;
     return launch_grouped_dt<MODE_DGRAD2>(act_dtype, a, (hipStream_t)stream);
 }
 
@@ -1299,6 +1302,7 @@ extern "C" int mx_experts_combine(const void *y, int64_t ldy, const int32_t *ord
     if (T == 0 || N == 0) return MX_OK;
     if (N % 8 || !aligned(y, 16) || !aligned(out, 16) || ldy % 8 || ldo % 8) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     const int64_t pairs = T * top_k;
     if (order) {  // order == NULL: inv already holds the positions of this routing (an earlier call filled it)
         fill_i32_kernel<<<dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st>>>(inv, pairs, -1);
@@ -1319,7 +1323,7 @@ extern "C" int mx_experts_combine(const void *y, int64_t ldy, const int32_t *ord
 }
 
 template <int CDT>
-static int launch_wgrad(WgradArgs a, hipStream_t st) {
+static int launch_wgrad(WgradArgs a, float *ws, int64_t ws_bytes, hipStream_t st) {
     typedef Big S;
     a.tiles_m = (a.N + S::BM - 1) / S::BM;
     a.tiles_n = (a.Kout + S::BN - 1) / S::BN;
@@ -1330,17 +1334,18 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
     const int cus = num_cus();
     // With more tile ids than workgroups the K split can still pay: the ids of experts without
     // rows are empty, and how many those are is only known on the device.
-    a.ws = work < (1 << 27) ? mx::split_scratch(st, cus, (size_t)S::BM * S::BN) : nullptr;
+    const bool fits = ws && !((uintptr_t)ws & 15) && ws_bytes >= 2 * (int64_t)cus * S::BM * S::BN * (int64_t)sizeof(float);
+    a.ws = work < (1 << 27) && fits ? ws : nullptr;  // two fp32 tile slots per workgroup, or whole tiles only
     a.slots = a.ws ? 2 * cus : 0;
     dim3 grid((unsigned)(work * (a.slots ? 8 : 1) < cus ? work * (a.slots ? 8 : 1) : cus)), block(S::NTHR);
     // scale rows with 12 readable bytes behind their last stage take one 16-byte fetch per four stages
     const bool quad = a.ldas >= a.KB + 12 && a.ldbs >= a.KB + 12;
-    auto kern = quad ? grouped_wgrad_kernel<S, CDT, SCALES_QUAD> : grouped_wgrad_kernel<S, CDT, SCALES_DWORD>;
-    if (!allow_dynamic_lds((const void *)kern, S::LDS_BYTES)) return MX_ELAUNCH;
     const int chunks = (a.N + 63) / 64;
     if ((int64_t)a.E * chunks >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
     wgrad_zero_kernel<CDT><<<dim3((unsigned)(a.E * chunks)), dim3(256), 0, st>>>(a, chunks);
-    kern<<<grid, block, S::LDS_BYTES, st>>>(a);
+    const int rc = quad ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_QUAD>>(grid, block, S::LDS_BYTES, st, a)
+                        : launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
+    if (rc != MX_OK) return rc;
     // tiles are only split while (tiles x slices) fit the 2 * cus slots, so 4 * cus workgroups cover every unit at once
     const int64_t units = work * S::MT < 4 * (int64_t)cus ? work * S::MT : 4 * (int64_t)cus;
     if (a.slots) wgrad_reduce_kernel<S, CDT><<<dim3((unsigned)units), block, 0, st>>>(a, (int)grid.x);
@@ -1350,9 +1355,9 @@ static int launch_wgrad(WgradArgs a, hipStream_t st) {
 extern "C" int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t lda, int64_t ldas, const uint8_t *bq,
                                    const uint8_t *bs, int64_t ldb, int64_t ldbs, const int32_t *offsets, int64_t E,
                                    int64_t M, void *dw, int dw_dtype, int64_t stride_dwe, int64_t lddw, int64_t N,
-                                   int64_t Kout, void *stream) {
+                                   int64_t Kout, void *workspace, int64_t workspace_bytes, void *stream) {
     if (E <= 0 || E >= (1 << 20) || M < 0 || M >= 0x7FFFFFFF || N < 0 || Kout < 0 || N >= 0x7FFFFFFF ||
-        Kout >= 0x7FFFFFFF || lddw < Kout)
+        Kout >= 0x7FFFFFFF || lddw < Kout || workspace_bytes < 0)
         return MX_EINVAL;
     const int64_t mpad = ((M + 127) / 128 + E) * 128;
     if (lda < mpad || ldb < mpad || ldas < mpad / MX_BLOCK || ldbs < mpad / MX_BLOCK) return MX_EINVAL;
@@ -1365,10 +1370,11 @@ extern "C" int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t
     a.dw = dw, a.stride_dwe = stride_dwe, a.lddw = lddw, a.offsets = offsets, a.E = (int)E, a.N = (int)N,
     a.Kout = (int)Kout, a.KB = (int)(mpad / MX_BLOCK);
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     switch (dw_dtype) {
-    case MX_BF16: return launch_wgrad<MX_BF16>(a, st);
-    case MX_FP16: return launch_wgrad<MX_FP16>(a, st);
-    case MX_FP32: return launch_wgrad<MX_FP32>(a, st);
+    case MX_BF16: return launch_wgrad<MX_BF16>(a, (float *)workspace, workspace_bytes, st);
+    case MX_FP16: return launch_wgrad<MX_FP16>(a, (float *)workspace, workspace_bytes, st);
+    case MX_FP32: return launch_wgrad<MX_FP32>(a, (float *)workspace, workspace_bytes, st);
     default: return MX_EINVAL;
     }
 }

@@ -303,6 +303,7 @@ extern "C" int mx_rmsnorm_quantize(const void *x, int x_dtype, int64_t M, int64_
         return MX_EUNSUPPORTED;
     NormArgs a = {x, weight, out, rstd, q, s, M, ldx, ldo, ldq, lds, (int)K, eps};
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     switch (x_dtype) {
     case MX_BF16: return launch_norm_w<MX_BF16>(a, w_dtype, st);
     case MX_FP16: return launch_norm_w<MX_FP16>(a, w_dtype, st);
@@ -336,6 +337,7 @@ extern "C" int mx_rmsnorm_backward(const void *x, int dtype, int64_t M, int64_t 
         return MX_EUNSUPPORTED;
     NormBwdArgs a = {x, weight, dout, rstd, dx, dw_part, M, ldx, lddo, lddx, (int)K};
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     const bool w32 = weight && w_dtype == MX_FP32;
     if (weight && !w32 && w_dtype != dtype) return MX_EUNSUPPORTED;
     if (dtype == MX_BF16) return w32 ? launch_norm_bwd<MX_BF16, MX_FP32>(a, parts, st) : launch_norm_bwd<MX_BF16, MX_BF16>(a, parts, st);

@@ -790,6 +790,7 @@ extern "C" int mx_quantize_cols(const void *x, int x_dtype, int64_t M, int64_t K
     if (M < 0 || K < 0 || M % MX_BLOCK || ldx < K || ldqT < M || ldsT < M / MX_BLOCK) return MX_EINVAL;
     if (M == 0 || K == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     if (!cols_vec_ok(x, x_dtype, K, ldx, qT, ldqT)) {
         // Rows of the transposed view, one thread per block.
         switch (x_dtype) {
@@ -812,6 +813,7 @@ extern "C" int mx_quantize_rows(const void *x, int x_dtype, int64_t M, int64_t K
     if (M < 0 || K < 0 || K % MX_BLOCK || ldq < K || lds < K / MX_BLOCK) return MX_EINVAL;
     if (M == 0 || K == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     // A transposed view (unit stride down the rows) is the column quantizer of the
     // matrix underneath it: no copy is made.
     if (sx_col != 1 && sx_row == 1 && M > 1 && cols_vec_ok(x, x_dtype, M, sx_col, q, ldq))
@@ -849,6 +851,7 @@ extern "C" int mx_quantize_heads(const void *x, int x_dtype, int64_t T, int64_t 
         (mu && !aligned(mu, 16)) || T * (H * D / 8) >= (int64_t)0x7FFFFF00)
         return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     switch (x_dtype) {
     case MX_BF16: return launch_heads<MX_BF16>(x, T, H, D, stride_t, stride_h, mu, q, s, st);
     case MX_FP16: return launch_heads<MX_FP16>(x, T, H, D, stride_t, stride_h, mu, q, s, st);
@@ -865,6 +868,7 @@ extern "C" int mx_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K
         return MX_EINVAL;
     if (M == 0 || K == 0) return MX_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     if (!cols_vec_ok(x, x_dtype, K, ldx, qT, ldqT) || !aligned(q, 8) || ldq % 8) {
         if (panels) return MX_EUNSUPPORTED;
         int rc = mx_quantize_rows(x, x_dtype, M, K, ldx, 1, q, ldq, s, lds, stream);
@@ -891,6 +895,7 @@ extern "C" int mx_quantize_dual_batch(const mx_quant_problem *problems, int coun
         if (p.M && p.K && (!p.x || !p.q || !p.s || !p.qT || !p.sT)) return MX_EINVAL;
     }
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     QuantBatchArgs b;
     b.count = 0;
     int64_t total = 0;
@@ -954,6 +959,7 @@ extern "C" int mx_swiglu_quantize_rows(const void *gate, const void *up, int dty
         M * (K / 8) >= (int64_t)0x7FFFFF00)
         return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     return dtype == MX_BF16 ? launch_swiglu<MX_BF16>(gate, up, M, K, ldg, ldu, q, ldq, s, lds, st)
                             : launch_swiglu<MX_FP16>(gate, up, M, K, ldg, ldu, q, ldq, s, lds, st);
 }
@@ -972,6 +978,7 @@ extern "C" int mx_swiglu_quantize_dual(const void *gu, int dtype, int64_t M, int
     dim3 grid((unsigned)((H + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
     if (grid.y > 65535u) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, 0, panels ? H * 128 : 0);
     if (dtype == MX_BF16) swiglu_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(gu, M, H, ldgu, o);
     else swiglu_quant_dual_kernel<MX_FP16><<<grid, dim3(256), 0, st>>>(gu, M, H, ldgu, o);
@@ -995,6 +1002,7 @@ extern "C" int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const v
     dim3 grid((unsigned)((H + QC_TILE - 1) / QC_TILE), (unsigned)((M + QC_TILE - 1) / QC_TILE));
     if (grid.y > 65535u) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, q_panels ? M * 128 : 0, qt_panels ? 2 * H * 128 : 0);
     if (H % 128) o.pack_row_scales = 0;  // the up half's scale columns start at H/32: keep dword stores aligned
     if (dtype == MX_BF16) swiglu_bwd_quant_dual_kernel<MX_BF16><<<grid, dim3(256), 0, st>>>(dh, lddh, gu, ldgu, M, H, o);
@@ -1025,6 +1033,7 @@ extern "C" int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, i
     a.span = ctiles >= 4 && (int64_t)tiles * (ctiles / 4) >= 2 * (int64_t)mx::num_cus() ? 4 : 1;
     dim3 grid((unsigned)((ctiles + a.span - 1) / a.span), (unsigned)tiles);
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
 #define MX_QCG_LAUNCH(DT, SRC)                                                                     \
     do {                                                                                           \
         if (a.span > 1) quant_cols_grouped_walk_kernel<DT, SRC><<<grid, dim3(256), 0, st>>>(a, o, mpad); \
@@ -1082,6 +1091,7 @@ static int swizzle_launch(bool to_swizzled, uint8_t *natural, int64_t lds, uint8
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7FFFFFFF) return MX_EUNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     if (to_swizzled)
         mx::swizzle_scales_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(natural, lds, swizzled, rows, cols,
                                                                                     col_tiles, total);

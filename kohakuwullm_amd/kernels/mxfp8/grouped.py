@@ -167,10 +167,11 @@ def grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets, rows: int, out_dtype=torch.
     if atq.shape[1] != mpad or btq.shape[1] != mpad:
         raise ValueError(f"operands must span the padded token axis {mpad}, got {tuple(atq.shape)}, {tuple(btq.shape)}")
     dw = torch.empty(num_experts, n, k, device=atq.device, dtype=out_dtype)
+    ws = _lib.gemm_workspace(atq)
     _lib.invoke(
         "mx_grouped_wgrad_nt", 2.0 * rows * n * k, atq,
         atq.data_ptr(), ats.data_ptr(), atq.stride(0), ats.stride(0), btq.data_ptr(), bts.data_ptr(), btq.stride(0),
         bts.stride(0), offsets.data_ptr(), num_experts, rows, dw.data_ptr(), _lib.MX_DTYPE[out_dtype],
-        dw.stride(0), dw.stride(1), n, k,
+        dw.stride(0), dw.stride(1), n, k, ws.data_ptr(), ws.numel(),
     )
     return dw

@@ -10,8 +10,9 @@ follow autocast, never the weight.
 
 One difference from the reference, on purpose: WGRAD also runs in MXFP8
 (``dW = Qcol(dY) . Qcol(X)^T`` with 32-token blocks), where the reference multiplies in
-16 bits (``linear.py:72-73``).  It falls back to that 16-bit product only when the token
-count is not a multiple of 32.
+16 bits (``linear.py:72-73``).  A token count that is not a multiple of 32 is padded with
+zero rows in front of the quantizers: zero rows add nothing to ``dW``, and their rows of
+the output and of ``dX`` are dropped.
 """
 
 from __future__ import annotations
@@ -57,6 +58,12 @@ class _PadLastAxis:
         return F.pad(tensor, (0, self.width)) if self.width else tensor
 
 
+def pad_tokens(x2d: torch.Tensor) -> torch.Tensor:
+    """``x2d`` with zero rows appended up to the next multiple of 32 tokens (itself when it already is one)."""
+    extra = -x2d.shape[0] % BLOCK_SCALE
+    return F.pad(x2d, (0, 0, 0, extra)) if extra else x2d
+
+
 class _MXFP8Linear(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, wq_f, ws_f, wq_d, ws_d, pad_k):
@@ -65,21 +72,20 @@ class _MXFP8Linear(torch.autograd.Function):
         x2d = x.reshape(-1, shape[-1]).to(compute)
         if x2d.stride(-1) != 1:
             x2d = x2d.contiguous()
-        need_dw = ctx.needs_input_grad[1]
-        fp8_wgrad = need_dw and x2d.shape[0] % BLOCK_SCALE == 0 and x2d.shape[0] > 0
+        tokens = x2d.shape[0]
+        need_dw = ctx.needs_input_grad[1] and tokens > 0
         # WGRAD contracts over the tokens (tens of thousands): its operands are written stage-major, a
         # K stage of a tile in one contiguous run, when tokens come in whole panels and dout needs no padding
-        stage_major = fp8_wgrad and stage_major_ok(x2d.shape[0]) and pad_k.width == 0
-        if fp8_wgrad:
-            # One pass over x gives FPROP's operand and WGRAD's (blocks along tokens).
-            xq, xs, xtq, xts = quantize_mx_dual(x2d, stage_major_t=stage_major)
+        stage_major = need_dw and stage_major_ok(tokens) and pad_k.width == 0
+        if need_dw:
+            # One pass over x gives FPROP's operand and WGRAD's (blocks of 32 along the tokens).
+            xq, xs, xtq, xts = quantize_mx_dual(pad_tokens(x2d), stage_major_t=stage_major)
             saved_x = (xtq, xts)
         else:
             xq, xs = quantize_mx(x2d)
-            saved_x = (x2d if need_dw else None, None)
-        out = mxfp8_matmul_pq(xq, xs, wq_f, ws_f, compute)
+            saved_x = (None, None)
+        out = mxfp8_matmul_pq(xq, xs, wq_f, ws_f, compute)[:tokens]
         ctx.save_for_backward(*saved_x, wq_d, ws_d)
-        ctx.fp8_wgrad = fp8_wgrad
         ctx.stage_major = stage_major
         ctx.pad_k = pad_k
         ctx.x_dtype = x.dtype
@@ -89,28 +95,31 @@ class _MXFP8Linear(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout):
-        x_a, x_b, wq_d, ws_d = ctx.saved_tensors
+        xtq, xts, wq_d, ws_d = ctx.saved_tensors
         shape = dout.shape
         d2d = dout.reshape(-1, shape[-1]).to(ctx.compute).contiguous()
-        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        tokens = d2d.shape[0]
+        need_dx, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1] and xtq is not None
         dx = dw = None
         padded = ctx.pad_k(d2d)
-        if need_dw and ctx.fp8_wgrad:
-            dq, ds, dtq, dts = quantize_mx_dual(padded, stage_major_t=ctx.stage_major)
+        if need_dw:
+            dq, ds, dtq, dts = quantize_mx_dual(pad_tokens(padded), stage_major_t=ctx.stage_major)
             n = ctx.out_features
             # dW (out,in) = dY^T (out,tokens) . (X^T (in,tokens))^T, contraction over tokens.
-            wgrad = (dtq if ctx.stage_major else dtq[:n], dts[:n], x_a, x_b)
+            wgrad = (dtq if ctx.stage_major else dtq[:n], dts[:n], xtq, xts)
             if need_dx and ctx.x_dtype == ctx.compute:
                 # few tiles with a long K beside many with a short one: one launch shares the GPU
                 dx, dw = mxfp8_matmul_pq_batch([(dq, ds, wq_d, ws_d), wgrad], ctx.compute)
+                dx = dx[:tokens]
                 return dx.reshape(*shape[:-1], dx.shape[-1]), dw, None, None, None, None, None
             dw = mxfp8_matmul_pq(*wgrad, ctx.compute)
+        elif ctx.needs_input_grad[1]:
+            dw = torch.zeros(ctx.out_features, wq_d.shape[0], device=d2d.device, dtype=ctx.compute)  # no tokens
+            dq, ds = quantize_mx(padded) if need_dx else (None, None)
         else:
             dq, ds = quantize_mx(padded) if need_dx else (None, None)
-            if need_dw:
-                dw = d2d.t() @ x_a
         if need_dx:
-            dx = mxfp8_matmul_pq(dq, ds, wq_d, ws_d, ctx.x_dtype)
+            dx = mxfp8_matmul_pq(dq, ds, wq_d, ws_d, ctx.x_dtype)[:tokens]
             dx = dx.reshape(*shape[:-1], dx.shape[-1])
         return dx, dw, None, None, None, None, None
 

@@ -18,7 +18,7 @@ from __future__ import annotations
 import torch
 
 from kohakuwullm_amd import _lib
-from kohakuwullm_amd.kernels.mxfp8.linear import compute_dtype
+from kohakuwullm_amd.kernels.mxfp8.linear import compute_dtype, pad_tokens
 from kohakuwullm_amd.kernels.mxfp8.quantize import (
     BLOCK_SCALE,
     PANEL,
@@ -123,9 +123,11 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         x2d = x.reshape(-1, shape[-1]).to(compute)
         if x2d.stride(-1) != 1:
             x2d = x2d.contiguous()
+        tokens = x2d.shape[0]
+        x2d = pad_tokens(x2d)  # whole 32-token blocks for WGRAD; zero rows change no gradient
         # The operands of the three backward products that go down in one launch (contractions of
         # 8192 and 16384) are written stage-major: each K stage of a tile is then one contiguous run.
-        sm = x.dtype == compute and stage_major_ok(x2d.shape[0]) and stage_major_ok(w_out.shape[1])
+        sm = x.dtype == compute and stage_major_ok(tokens) and stage_major_ok(w_out.shape[1])
         xq, xs, xtq, xts = quantize_mx_dual(x2d, stage_major_t=sm)
         # GEMM, then one bandwidth-bound pass for SwiGLU and both casts: measured faster at the
         # benchmark shape (220 + 89 us) than the same work in the GEMM's epilogue
@@ -138,14 +140,15 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
             ctx.compute = compute
             ctx.x_dtype = x.dtype
             ctx.stage_major = sm
-        return y.reshape(*shape[:-1], y.shape[-1])
+        return y[:tokens].reshape(*shape[:-1], y.shape[-1])
 
     @staticmethod
     def backward(ctx, dout):
         xtq, xts, gu, htq, hts, win_dq, win_ds, wout_dq, wout_ds = ctx.saved_tensors
         shape = dout.shape
         d2d = dout.reshape(-1, shape[-1]).to(ctx.compute).contiguous()
-        dq, ds, dtq, dts = quantize_mx_dual(d2d, stage_major_t=ctx.stage_major)
+        tokens = d2d.shape[0]
+        dq, ds, dtq, dts = quantize_mx_dual(pad_tokens(d2d), stage_major_t=ctx.stage_major)
         dh = mxfp8_matmul_pq(dq, ds, wout_dq, wout_ds, ctx.compute)
         pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu, stage_major=ctx.stage_major)
         # The last three products are independent and none fills the GPU alone (dW has few
@@ -166,7 +169,7 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
                     grads[i] = mxfp8_matmul_pq(*w, ctx.x_dtype if i == 0 else ctx.compute)
         dx, dw_in, dw_out = grads
         if dx is not None:
-            dx = dx.reshape(*shape[:-1], -1)
+            dx = dx[:tokens].reshape(*shape[:-1], -1)
         return dx, dw_in, dw_out, None, None, None, None
 
 
@@ -176,11 +179,9 @@ def mxfp8_swiglu_mlp(x, w_in, w_out, packed) -> torch.Tensor:
     ``packed`` is ``(in_fwd, in_dgrad, out_fwd, out_dgrad)``, each a ``(codes, scales)`` pair:
     the weights blocked along their contraction axis for FPROP and along the other axis for
     DGRAD.  ``w_in``/``w_out`` are passed so autograd routes ``dW`` to the master parameters.
-    Tokens, ``dim`` and ``H`` must be multiples of 32.
+    ``dim`` and ``H`` must be multiples of 32; any token count is taken (it is padded with zero
+    rows to whole 32-token blocks, which changes no result).
     """
-    tokens = x.numel() // x.shape[-1]
-    if tokens % BLOCK_SCALE:
-        raise ValueError(f"token count {tokens} must be a multiple of {BLOCK_SCALE} for the MXFP8 WGRAD")
     if w_in.shape[0] != 2 * w_out.shape[1] or w_in.shape[1] != x.shape[-1] or w_out.shape[0] != x.shape[-1]:
         raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w_in {tuple(w_in.shape)}, w_out {tuple(w_out.shape)}")
     return _MXFP8SwiGLUMLP.apply(x, w_in, w_out, *packed)

@@ -168,11 +168,12 @@ def quantize_mx_dual_batch(xs: list[torch.Tensor]) -> list[tuple[torch.Tensor, t
 def _gemm_nt_into(aq, a_scale, bq, b_scale, out) -> None:
     m, k = aq.shape
     n = bq.shape[0]
+    ws = _lib.gemm_workspace(aq)
     _lib.invoke(
         "mx_gemm_nt", 2.0 * m * n * k, aq,
         aq.data_ptr(), a_scale.data_ptr(), bq.data_ptr(), b_scale.data_ptr(), out.data_ptr(),
         _lib.MX_DTYPE[out.dtype], m, n, k, aq.stride(0), a_scale.stride(0), bq.stride(0), b_scale.stride(0),
-        out.stride(0), 0,
+        out.stride(0), 0, ws.data_ptr(), ws.numel(),
     )
 
 
@@ -262,7 +263,9 @@ def mxfp8_matmul_pq_batch(problems, out_dtype: torch.dtype = torch.bfloat16) -> 
         d.lda = PANEL if ts[0].dim() == 3 else ts[0].stride(0)
         d.ldb = PANEL if ts[2].dim() == 3 else ts[2].stride(0)
         d.ldas, d.ldbs, d.ldc = ts[1].stride(0), ts[3].stride(0), n
-    _lib.invoke("mx_gemm_nt_batch", flops, outs[0], ctypes.addressof(descs), len(problems), _lib.MX_DTYPE[out_dtype])
+    ws = _lib.gemm_workspace(outs[0])
+    _lib.invoke("mx_gemm_nt_batch", flops, outs[0], ctypes.addressof(descs), len(problems), _lib.MX_DTYPE[out_dtype],
+                ws.data_ptr(), ws.numel())
     return outs
 
 

@@ -47,7 +47,12 @@ BUCKETS = ("fp8", "skipped", "unreached", "never")
 
 @dataclass
 class SwapReport:
-    """What the surgery converted, refused and could not reach, with a per-token MAC census."""
+    """What the surgery converted, refused and could not reach, with a per-token MAC census.
+
+    Field names and meaning are the reference's (``mxfp8_swap.py:41-103``): ``swapped`` names tensors,
+    ``modules`` the modules that hold an fp8 cache (what ``refresh_mxfp8_weights`` counts); ``skipped``,
+    ``unreached`` and ``unaccounted`` block a run, ``by_design`` and ``out_of_scope`` do not.
+    """
 
     swapped: list[str] = field(default_factory=list)
     modules: list[str] = field(default_factory=list)
@@ -60,31 +65,35 @@ class SwapReport:
 
     @property
     def blocking(self) -> bool:
-        return bool(self.skipped or self.unreached or self.unaccounted)
+        return any((self.skipped, self.unreached, self.unaccounted))
 
     @property
     def total_mac(self) -> int:
         return sum(self.mac.values())
 
     def share(self, bucket: str) -> float:
-        total = self.total_mac
-        return self.mac[bucket] / total if total else 0.0
+        return self.mac[bucket] / self.total_mac if self.total_mac else 0.0
 
     def summary(self) -> str:
-        lines = [
-            f"MXFP8: {len(self.swapped)} tensor(s) in fp8 over {len(self.modules)} module(s), "
-            f"{self.share('fp8'):.1%} of {self.total_mac / 1e6:.1f}M per-token MAC"
-        ]
-        for label, entries in (("SKIPPED", self.skipped), ("UNREACHED", self.unreached)):
-            lines += [f"  {label} {name}: {reason}" for name, reason in entries]
-        if self.unaccounted:
-            lines.append(f"  UNACCOUNTED: {', '.join(self.unaccounted)}")
-        if self.by_design:
-            lines.append(f"  bf16 by design: {len(self.by_design)} tensor(s), {self.share('never'):.1%} of per-token MAC")
-        return "\n".join(lines)
+        """A few lines for a log: the fp8 share first, then every finding that blocks, then what stays 16-bit on purpose."""
+        out = [f"MXFP8 swap: {len(self.swapped)} tensors / {len(self.modules)} modules now fp8 = "
+               f"{self.share('fp8'):.1%} of {self.total_mac / 1e6:.1f}M MAC per token"]
+        findings = [("skipped", name, why) for name, why in self.skipped]
+        findings += [("unreached", name, why) for name, why in self.unreached]
+        findings += [("unaccounted", name, "a matmul-shaped parameter nobody declared") for name in self.unaccounted]
+        out += [f"  BLOCKING [{kind}] {name}: {why}" for kind, name, why in findings]
+        for bucket in ("skipped", "unreached"):
+            if self.mac[bucket]:
+                out.append(f"  {bucket}: {self.mac[bucket] / 1e6:.1f}M MAC per token ({self.share(bucket):.1%})")
+        kept = len(self.by_design) + len(self.out_of_scope)
+        if kept:
+            out.append(f"  16-bit on purpose: {len(self.by_design)} by design, {len(self.out_of_scope)} out of scope "
+                       f"({self.share('never'):.1%} of MAC)")
+        return "\n".join(out)
 
 
 def _reject(module: nn.Linear) -> str | None:
+    """Why ``MXFP8Linear`` cannot stand in for this layer (the reference's two rules and wording, ``mxfp8_swap.py:106-113``)."""
     if module.bias is not None:
         return "has a bias; MXFP8Linear is bias-free"
     if module.in_features % 128:
@@ -92,116 +101,131 @@ def _reject(module: nn.Linear) -> str | None:
     return None
 
 
-def _qualify(prefix: str, name: str) -> str:
+class _Census:
+    """The report under construction plus the set of parameters somebody has answered for."""
+
+    def __init__(self, scope) -> None:
+        self.report = SwapReport()
+        self.scope = scope
+        self._claimed: set[int] = set()
+
+    def claim(self, tensor) -> None:
+        self._claimed.add(id(tensor))
+
+    def claimed(self, tensor) -> bool:
+        return id(tensor) in self._claimed
+
+    def wanted(self, qualified: str) -> bool:
+        return self.scope is None or any(part in qualified for part in self.scope)
+
+    def book(self, outcome: str, name: str, mac: int, why: str | None = None) -> None:
+        """Enter one tensor under one of: fp8, skipped, unreached, by_design, out_of_scope."""
+        r = self.report
+        if outcome == "fp8":
+            r.swapped.append(name)
+        elif outcome == "skipped":
+            r.skipped.append((name, why))
+        elif outcome == "unreached":
+            r.unreached.append((name, why))
+        elif outcome == "by_design":
+            r.by_design.append(name)
+        else:
+            r.out_of_scope.append(name)
+        r.mac[outcome if outcome in BUCKETS else "never"] += mac
+
+
+def _join(prefix: str, name: str) -> str:
     return f"{prefix}.{name}" if prefix else name
 
 
-def _in_scope(qualified: str, scope) -> bool:
-    return scope is None or any(part in qualified for part in scope)
-
-
-def _swap_children(parent, prefix, linear_cls, report, accounted, scope) -> None:
-    for name in PROJECTION_NAMES:
-        child = getattr(parent, name, None)
-        if not isinstance(child, (nn.Linear, linear_cls)):
+def _convert_linears(parent: nn.Module, prefix: str, linear_cls: type, census: _Census) -> None:
+    """The projection-named ``nn.Linear`` children of ``parent``: replace the ones ``linear_cls`` can stand in for."""
+    for name, child in list(parent.named_children()):
+        if name not in PROJECTION_NAMES or not isinstance(child, (nn.Linear, linear_cls)):
             continue
-        qualified = _qualify(prefix, name)
-        mac = child.in_features * child.out_features
-        accounted.add(id(child.weight))
-        if isinstance(child, linear_cls):  # a second swap over the same model
-            report.swapped.append(qualified)
-            report.modules.append(qualified)
-            report.mac["fp8"] += mac
-            continue
-        if not _in_scope(qualified, scope):
-            report.out_of_scope.append(qualified)
-            report.mac["never"] += mac
-            continue
-        reason = _reject(child)
-        if reason is not None:
-            report.skipped.append((qualified, reason))
-            report.mac["skipped"] += mac
-            continue
-        replacement = linear_cls(child.in_features, child.out_features, dtype=child.weight.dtype)
-        with torch.no_grad():
-            replacement.weight.copy_(child.weight)
-        replacement.to(child.weight.device)
-        setattr(parent, name, replacement)
-        accounted.add(id(replacement.weight))
-        report.swapped.append(qualified)
-        report.modules.append(qualified)
-        report.mac["fp8"] += mac
+        where, mac = _join(prefix, name), child.in_features * child.out_features
+        census.claim(child.weight)
+        if isinstance(child, linear_cls):  # converted by an earlier swap of the same model
+            outcome, why = "fp8", None
+        elif not census.wanted(where):
+            outcome, why = "out_of_scope", None
+        else:
+            why = _reject(child)
+            outcome = "skipped" if why else "fp8"
+        if outcome == "fp8" and not isinstance(child, linear_cls):
+            stand_in = linear_cls(child.in_features, child.out_features, dtype=child.weight.dtype)
+            with torch.no_grad():
+                stand_in.weight.copy_(child.weight)  # the A/B arms must start from identical weights
+            setattr(parent, name, stand_in.to(child.weight.device))
+            census.claim(stand_in.weight)
+        census.book(outcome, where, mac, why)
+        if outcome == "fp8":
+            census.report.modules.append(where)
 
 
-def _resolve_attr(module: nn.Module, path: str):
-    obj = module
-    for part in path.split("."):
-        obj = getattr(obj, part)
-    return obj
-
-
-def _visit_declared(parent, prefix, report, accounted, convert_declared, scope) -> None:
-    declared: dict[str, Matmul] = {}
+def _declarations(parent: nn.Module) -> dict[str, Matmul]:
+    """What ``parent`` says about the matmuls it holds as bare parameters (an embedding speaks for itself)."""
+    said: dict[str, Matmul] = {}
     if isinstance(parent, nn.Embedding):
-        declared["weight"] = Matmul(0, "an embedding is a gather, not a GEMM", never=True)
+        said["weight"] = Matmul(0, "an embedding is a gather, not a GEMM", never=True)
     declare = getattr(parent, DECLARE, None)
-    if declare is not None:
-        declared.update(declare())
-    if not declared:
-        return
-    for name in declared:
-        accounted.add(id(_resolve_attr(parent, name)))
-    for name, entry in declared.items():
+    if callable(declare):
+        said.update(declare())
+    return said
+
+
+def _convert_declared(parent: nn.Module, prefix: str, census: _Census, convert_declared: bool) -> None:
+    """Account for the tensors ``parent`` declares; convert them when all that may go to fp8 can."""
+    said = _declarations(parent)
+    open_cases: list[tuple[str, Matmul]] = []
+    for name, entry in said.items():
+        tensor = parent
+        for part in name.split("."):  # a declaration may name a child's tensor ("router.weight")
+            tensor = getattr(tensor, part)
+        census.claim(tensor)
         if entry.never:
-            report.by_design.append(_qualify(prefix, name))
-            report.mac["never"] += entry.mac_per_token
-    live = {n: e for n, e in declared.items() if not e.never}
-    if not _in_scope(prefix, scope):
-        for name, entry in live.items():
-            report.out_of_scope.append(_qualify(prefix, name))
-            report.mac["never"] += entry.mac_per_token
+            census.book("by_design", _join(prefix, name), entry.mac_per_token)
+        else:
+            open_cases.append((_join(prefix, name), entry))
+    if not open_cases:
         return
-    blocked = {n: e for n, e in live.items() if e.refusal is not None}
-    eligible = {n: e for n, e in live.items() if e.refusal is None}
-    if blocked:
-        for name, entry in blocked.items():
-            report.skipped.append((_qualify(prefix, name), entry.refusal))
-            report.mac["skipped"] += entry.mac_per_token
-        for name, entry in eligible.items():
-            report.skipped.append((_qualify(prefix, name), f"a sibling tensor in {prefix or '<root>'} is refused"))
-            report.mac["skipped"] += entry.mac_per_token
-        return
-    if not eligible:
-        return
-    convert = getattr(parent, CONVERT, None) if convert_declared else None
-    if convert is None:
-        why = (f"{type(parent).__name__} declares it fp8-eligible but has no {CONVERT}()" if convert_declared
-               else "the caller passed convert_declared=False")
-        for name, entry in eligible.items():
-            report.unreached.append((_qualify(prefix, name), why))
-            report.mac["unreached"] += entry.mac_per_token
-        return
-    convert()
-    report.modules.append(prefix)
-    for name, entry in eligible.items():
-        report.swapped.append(_qualify(prefix, name))
-        report.mac["fp8"] += entry.mac_per_token
+    if not census.wanted(prefix):
+        verdict = lambda entry: ("out_of_scope", None)  # noqa: E731
+    elif any(entry.refusal for _, entry in open_cases):
+        # one refused tensor keeps the whole module in 16 bits; its siblings point at it
+        sibling = f"a sibling tensor in {prefix or '<root>'} is refused"
+        verdict = lambda entry: ("skipped", entry.refusal or sibling)  # noqa: E731
+    elif not convert_declared:
+        verdict = lambda entry: ("unreached", "the caller passed convert_declared=False")  # noqa: E731
+    elif not callable(getattr(parent, CONVERT, None)):
+        missing = f"{type(parent).__name__} declares it fp8-eligible but has no {CONVERT}()"
+        verdict = lambda entry: ("unreached", missing)  # noqa: E731
+    else:
+        getattr(parent, CONVERT)()
+        census.report.modules.append(prefix)
+        verdict = lambda entry: ("fp8", None)  # noqa: E731
+    for where, entry in open_cases:
+        outcome, why = verdict(entry)
+        census.book(outcome, where, entry.mac_per_token, why)
 
 
 def swap_mxfp8(model: nn.Module, linear_cls: type = MXFP8Linear, convert_declared: bool = True,
                scope: tuple[str, ...] | None = None) -> SwapReport:
-    """Convert every reachable matmul of ``model`` to MXFP8, in place; weights are copied."""
-    report = SwapReport()
-    accounted: set[int] = set()
+    """Convert every reachable matmul of ``model`` to MXFP8, in place; weights are copied.
+
+    ``scope``: substrings of qualified names to restrict the conversion to (the rest is reported as
+    ``out_of_scope`` and does not block).  ``convert_declared=False`` leaves declared bare-parameter
+    matmuls alone and reports them ``unreached``.  Signature and outcomes as ``mxfp8_swap.py:301-328``.
+    """
+    census = _Census(scope)
     for prefix, parent in list(model.named_modules()):
         if isinstance(parent, linear_cls):
             continue
-        _swap_children(parent, prefix, linear_cls, report, accounted, scope)
-        _visit_declared(parent, prefix, report, accounted, convert_declared, scope)
-    for name, param in model.named_parameters():
-        if param.dim() >= 2 and id(param) not in accounted:
-            report.unaccounted.append(f"{name}{tuple(param.shape)}")
-    return report
+        _convert_linears(parent, prefix, linear_cls, census)
+        _convert_declared(parent, prefix, census, convert_declared)
+    census.report.unaccounted += [f"{name}{tuple(p.shape)}" for name, p in model.named_parameters()
+                                  if p.dim() >= 2 and not census.claimed(p)]
+    return census.report
 
 
 def refresh_mxfp8_weights(model: nn.Module) -> int:

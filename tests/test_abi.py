@@ -29,7 +29,7 @@ def test_header_parses_to_the_expected_surface():
             "mx_quantize_cols_grouped", "mx_swiglu_quantize_rows", "mx_swiglu_quantize_dual",
             "mx_swiglu_bwd_quantize_dual", "mx_abi_version", "mx_strerror", "mx_device_supported",
             "mx_rmsnorm_quantize", "mx_rmsnorm_backward", "mx_expert_counts", "mx_expert_sort_workspace",
-            "mx_expert_sort", "mx_combine_routed", "mx_combine_routed_backward"} <= names
+            "mx_expert_sort", "mx_combine_routed", "mx_combine_routed_backward", "mx_gemm_workspace_bytes", "mx_gemm_nt_batch"} <= names
 
 
 def test_library_exports_every_declared_symbol():
@@ -50,8 +50,9 @@ def test_binding_matches_header():
     for name, (restype, argtypes) in _lib.SIGNATURES.items():
         assert len(argtypes) == declared[name], f"{name}: binding has {len(argtypes)} args, header {declared[name]}"
     lib = _lib.load()
-    assert lib.mx_abi_version() == 1
+    assert lib.mx_abi_version() == _lib.MX_ABI_VERSION == 2
     assert b"invalid" in lib.mx_strerror(-1) and lib.mx_strerror(0) == b"ok"
+    assert b"captured" in lib.mx_strerror(_lib.MX_ECAPTURE)
 
 
 def test_entry_points_validate_before_launch():
@@ -62,10 +63,13 @@ def test_entry_points_validate_before_launch():
     assert lib.mx_quantize_rows(None, 0, 4, 48, 48, 1, None, 48, None, 1, None) == _lib.MX_EINVAL  # K % 32
     assert lib.mx_quantize_cols(None, 0, 48, 64, 64, None, 48, None, 1, None) == _lib.MX_EINVAL  # M % 32
     assert lib.mx_quantize_rows(None, 0, 0, 64, 64, 1, None, 64, None, 2, None) == _lib.MX_OK  # empty
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 48, 48, 1, 48, 1, 4, 0, None) == _lib.MX_EINVAL
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 32, 2, 64, 2, 4, 0, None) == _lib.MX_EINVAL  # lda < K
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 64, 64, 2, 64, 2, 4, 0, None) == _lib.MX_OK
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 64, 2, 64, 2, 4, 1, None) == _lib.MX_EINVAL  # accumulate needs fp32
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 48, 48, 1, 48, 1, 4, 0, None, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 32, 2, 64, 2, 4, 0, None, 0, None) == _lib.MX_EINVAL  # lda < K
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 64, 64, 2, 64, 2, 4, 0, None, 0, None) == _lib.MX_OK
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 64, 2, 64, 2, 4, 1, None, 0, None) == _lib.MX_EINVAL  # accumulate needs fp32
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 64, 64, 2, 64, 2, 4, 0, None, -1, None) == _lib.MX_EINVAL  # workspace size
+    assert lib.mx_gemm_nt_batch(None, 0, 0, None, 0, None) == _lib.MX_OK and lib.mx_gemm_nt_batch(None, 1, 0, None, 0, None) == _lib.MX_EINVAL
+    assert lib.mx_grouped_wgrad_nt(None, None, 256, 8, None, None, 256, 8, None, 1, 128, None, 0, 0, 64, 64, 64, None, -1, None) == _lib.MX_EINVAL
     # expert dispatch: sizes, index widths and the workspace are checked before anything is launched
     assert lib.mx_expert_counts(None, 3, 8, 4, None, None) == _lib.MX_EINVAL  # idx_bytes
     assert lib.mx_expert_counts(None, 8, 8, 4, None, None) == _lib.MX_EINVAL  # null pointers
@@ -92,8 +96,8 @@ def test_entry_points_validate_before_launch():
     assert lib.mx_quantize_heads(None, 0, 0, 4, 64, 256, 64, None, None, None, None) == _lib.MX_OK
     assert lib.mx_quantize_heads(None, 0, 8, 4, 64, 256, 64, None, None, None, None) == _lib.MX_EINVAL  # null operands
     # a leading dimension of exactly 128 on a wider code matrix selects the stage-major layout: K % 128 then
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 256, 128, 8, 256, 8, 4, 0, None) == _lib.MX_OK  # A panels, empty
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 160, 128, 5, 160, 5, 4, 0, None) == _lib.MX_EINVAL  # K % 128
-    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 256, 64, 8, 256, 8, 4, 0, None) == _lib.MX_EINVAL  # lda < K, not 128
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 0, 4, 256, 128, 8, 256, 8, 4, 0, None, 0, None) == _lib.MX_OK  # A panels, empty
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 160, 128, 5, 160, 5, 4, 0, None, 0, None) == _lib.MX_EINVAL  # K % 128
+    assert lib.mx_gemm_nt(None, None, None, None, None, 0, 4, 4, 256, 64, 8, 256, 8, 4, 0, None, 0, None) == _lib.MX_EINVAL  # lda < K, not 128
     assert lib.mx_quantize_dual(None, 0, 0, 64, 64, None, 64, None, 2, None, 128, None, 0, None) == _lib.MX_OK
     assert lib.mx_quantize_dual(None, 0, 160, 64, 64, None, 64, None, 2, None, 128, None, 5, None) == _lib.MX_EINVAL  # panels need M % 128

@@ -269,12 +269,12 @@ def test_gemm_split_k_accumulate(oracle):
     for split in (1, 4, 7):
         c = base.clone()
         _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(),
-                    _lib.MX_DTYPE[torch.float32], m, n, k, k, k // 32, k, k // 32, n, 1 | (split << 8))
+                    _lib.MX_DTYPE[torch.float32], m, n, k, k, k // 32, k, k // 32, n, 1 | (split << 8), None, 0)
         assert oracle.rel_error((c - base).cpu(), ref) < TOL_FP32, split
     c16 = torch.zeros(m, n, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(ValueError):  # accumulation is fp32 only
         _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c16.data_ptr(),
-                    _lib.MX_DTYPE[torch.bfloat16], m, n, k, k, k // 32, k, k // 32, n, 1)
+                    _lib.MX_DTYPE[torch.bfloat16], m, n, k, k, k // 32, k, k // 32, n, 1, None, 0)
 
 
 def test_gemm_errors():
@@ -332,3 +332,40 @@ def test_gemm_split_on_two_streams(oracle):
         for out in outs[i]:
             assert torch.equal(out, outs[i][0])
         assert oracle.rel_error(outs[i][0].cpu(), refs[i]) < TOL_FP32
+
+
+@pytest.mark.parametrize("m,n,k", [(1536, 4096, 16384), (768, 512, 8192), (16384, 1536, 4096)])
+def test_workspace_is_the_callers(oracle, m, n, k):
+    """Shapes whose last round of tiles is sparse: with the caller's workspace the K stages of those tiles are
+    split, without one (NULL, or too small) every tile is computed whole.  Same product either way, and the
+    library never allocates: a poisoned workspace one byte short is not touched."""
+    from kohakuwullm_amd import _lib
+
+    aq, as_, bq, bs = _operands(oracle, m, n, k)
+    f8 = torch.float8_e4m3fn
+    a, sa, b, sb = aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)
+    need = int(_lib.load().mx_gemm_workspace_bytes())
+    assert need == 2 * torch.cuda.get_device_properties(0).multi_processor_count * 256 * 256 * 4
+
+    def run(ws, nbytes):
+        c = torch.full((m, n), float("nan"), device=DEV, dtype=torch.bfloat16)
+        _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(),
+                    _lib.MX_DTYPE[torch.bfloat16], m, n, k, k, k // 32, k, k // 32, n, 0, ws, nbytes)
+        return c
+
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)
+    split = run(ws.data_ptr(), need)
+    whole = run(None, 0)
+    short = run(ws.data_ptr(), need - 1)
+    assert torch.equal(whole, short)
+    rows = torch.randperm(m, generator=torch.Generator().manual_seed(SEED))[:96]
+    ref = oracle.gemm_nt(aq[rows], as_[rows], bq, bs)
+    for got in (split, whole):
+        assert torch.isfinite(got.float()).all()
+        assert oracle.rel_error(got[rows.to(DEV)].cpu(), ref) < TOL_BF16
+    assert oracle.rel_error(split.cpu(), whole.double().cpu()) < 2e-3  # the same fp32 sums in another order
+    ws.fill_(0xA5)
+    run(ws.data_ptr(), need - 1)
+    torch.cuda.synchronize()
+    assert bool((ws == 0xA5).all())
+    assert torch.equal(_mx().mxfp8_matmul_pq(a, sa, b, sb), split)  # the wrapper brings a full workspace

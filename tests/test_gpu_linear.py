@@ -35,12 +35,11 @@ def _linear_refs(ora, x2d, w, dy2d, pad=0):
     dq, ds = ora.quantize_rows(dyp)
     wtq, wts = ora.quantize_rows(wtp)
     dx = ora.gemm_nt(dq, ds, wtq, wts)
-    if x2d.shape[0] % 32 == 0:
-        dtq, dts = ora.quantize_cols(dy2d)
-        xtq, xts = ora.quantize_cols(x2d)
-        dw = ora.gemm_nt(dtq, dts, xtq, xts)
-    else:
-        dw = dy2d.double().T @ x2d.double()
+    # token blocks of 32: a ragged last block is completed with zero rows, which add nothing to dW
+    extra = -x2d.shape[0] % 32
+    dtq, dts = ora.quantize_cols(torch.nn.functional.pad(dy2d, (0, 0, 0, extra)))
+    xtq, xts = ora.quantize_cols(torch.nn.functional.pad(x2d, (0, 0, 0, extra)))
+    dw = ora.gemm_nt(dtq, dts, xtq, xts)
     return y, dx, dw
 
 
@@ -155,7 +154,7 @@ def test_swap_and_refresh(oracle):
     assert rep.blocking and any("in_features=192" in why for _, why in rep.skipped)
 
 
-@pytest.mark.parametrize("tokens,dim,hidden", [(256, 256, 512), (128, 128, 96)])
+@pytest.mark.parametrize("tokens,dim,hidden", [(256, 256, 512), (128, 128, 96), (77, 128, 64)])
 def test_fused_swiglu_mlp(oracle, tokens, dim, hidden):
     from kohakuwullm_amd.kernels.mxfp8.mlp import mxfp8_swiglu_mlp
     from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx, quantize_mx_cols
@@ -178,8 +177,12 @@ def test_fused_swiglu_mlp(oracle, tokens, dim, hidden):
     sg = torch.sigmoid(g)
     dpre = torch.cat([dh * u * sg * (1 + g * (1 - sg)), dh * g * sg], dim=-1)
     dx_ref = ora.gemm_nt(*ora.quantize_rows(dpre), *ora.quantize_cols(w_in))
-    dwin_ref = ora.gemm_nt(*ora.quantize_cols(dpre), *ora.quantize_cols(x))
-    dwout_ref = ora.gemm_nt(*ora.quantize_cols(dy), *ora.quantize_cols(h))
+
+    def tok(t):  # the token axis in whole blocks of 32: zero rows complete a ragged last block
+        return torch.nn.functional.pad(t, (0, 0, 0, -t.shape[0] % 32))
+
+    dwin_ref = ora.gemm_nt(*ora.quantize_cols(tok(dpre)), *ora.quantize_cols(tok(x)))
+    dwout_ref = ora.gemm_nt(*ora.quantize_cols(tok(dy)), *ora.quantize_cols(tok(h)))
     assert ora.rel_error(y.detach().cpu(), y_ref) < TOL
     assert ora.rel_error(xd.grad.cpu(), dx_ref) < TOL
     assert ora.rel_error(wi.grad.cpu(), dwin_ref) < TOL

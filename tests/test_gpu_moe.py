@@ -495,13 +495,15 @@ def test_expert_call_contract():
 
 
 def test_moe_module_swap_and_train_step(oracle):
-    """MoEMLP through swap_mxfp8: declaration protocol, fused vs eager outputs, refresh contract."""
+    """MoEMLP built from a reference-style spec, through swap_mxfp8: declaration protocol, MXFP8 vs 16-bit outputs, refresh contract."""
     from kohakuwullm_amd.models.moe import MoEMLP, expert_sort
     from kohakuwullm_amd.models.mxfp8_swap import refresh_mxfp8_weights, swap_mxfp8
-    from kohakuwullm_amd.registry import MOE, build
+    from kohakuwullm_amd.registry import MLP, build
 
     torch.manual_seed(0)
-    moe = build("moe", MOE, dim=256, hidden=128, num_experts=8, top_k=2).to(DEV)
+    spec = {"name": "moe", "hidden": 128, "num_experts": 8, "top_k": 2, "num_shared": 0, "score_func": "softmax",
+            "bias_update_rate": 0.0}
+    moe = build(spec, MLP, dim=256).to(DEV, torch.bfloat16)
     x = torch.randn(4, 96, 256, device=DEV, dtype=torch.bfloat16)
     y_eager = moe(x)
     report = swap_mxfp8(moe)
@@ -521,13 +523,60 @@ def test_moe_module_swap_and_train_step(oracle):
     moe.float()
     assert moe._packed is None
     # the unfused path is selected before conversion
-    moe2 = MoEMLP(256, 128, 8, 2, mxfp8_expert_path="unfused").to(DEV)
+    moe2 = MoEMLP(256, hidden=128, num_experts=8, top_k=2, num_shared=0).to(DEV, torch.bfloat16)
+    moe2.mxfp8_expert_path = "unfused"
     swap_mxfp8(moe2)
     assert moe2._routed == moe2._routed_mxfp8_unfused and moe2(x).shape == x.shape
-    bad = MoEMLP(256, 48, 4, 2).to(DEV)
+    bad = MoEMLP(256, hidden=48, num_experts=4, top_k=2, num_shared=0).to(DEV)
     assert swap_mxfp8(bad).blocking
     # dispatch format: stable order inside an expert, offsets = cumsum(counts)
     idx = torch.tensor([2, 0, 2, 1, 0, 2], device=DEV)
     counts = torch.tensor([2, 1, 3], device=DEV, dtype=torch.int32)
     offsets, order, token_of, _ = expert_sort(idx, counts, 2, 3)
     assert offsets.tolist() == [0, 2, 3, 6] and order.tolist() == [1, 4, 3, 0, 2, 5] and token_of.tolist() == [0, 2, 1, 0, 1, 2]
+
+
+def test_moe_module_reference_defaults(oracle):
+    """The reference's defaults: one shared expert (a GLUMLP the swap converts too), sigmoid scores with the balancing
+    bias, master weights in fp32 under bf16 autocast, a router that reads another tensor, both MXFP8 paths."""
+    from kohakuwullm_amd.kernels.mxfp8.linear import MXFP8Linear
+    from kohakuwullm_amd.models.moe import MoEMLP
+    from kohakuwullm_amd.models.mxfp8_swap import refresh_mxfp8_weights, swap_mxfp8
+
+    torch.manual_seed(1)
+    moe = MoEMLP(256, hidden=128, num_experts=16, top_k=4, aux_loss_weight=0.01, z_loss_weight=1e-3).to(DEV)
+    assert moe.shared is not None and moe.shared.hidden == 128 and moe.num_buckets == 16 and not moe._has_sentinel
+    assert list(moe.state_dict()) == ["w_in", "w_out", "router.weight", "router.expert_bias", "router.load_accum",
+                                      "shared.w_in.weight", "shared.w_out.weight"]
+    assert moe.emits_router_loss and moe.active_parameters() == 4 * 3 * 128 * 256 + 16 * 256 + 3 * 128 * 256
+    x = torch.randn(200, 256, device=DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y16 = moe(x)
+    report = swap_mxfp8(moe)
+    assert not report.blocking, report.summary()
+    assert isinstance(moe.shared.w_in, MXFP8Linear) and isinstance(moe.shared.w_out, MXFP8Linear)
+    assert refresh_mxfp8_weights(moe) == 3  # the routed experts and the two shared projections
+    for path in ("fused", "unfused"):
+        moe.mxfp8_expert_path = path
+        moe.enable_mxfp8()
+        xg = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = moe(xg)
+            aux = moe.router_losses()
+        assert y.dtype == torch.bfloat16 and oracle.rel_error(y.float().cpu(), y16.float().cpu()) < 0.08, path
+        assert aux is not None and aux.requires_grad
+        (y.float().square().mean() + aux).backward()
+        assert moe.w_in.grad.dtype == torch.float32 and moe.w_in.grad.abs().sum() > 0 and xg.grad.abs().sum() > 0
+        assert moe.router.weight.grad.abs().sum() > 0 and moe.shared.w_in.weight.grad.abs().sum() > 0
+        moe.zero_grad()
+    # the balancing bias moves once per optimizer step and the load counter is cleared
+    stats = moe.router.update_bias()
+    assert stats.shape == (3,) and moe.router.load_accum.sum() == 0 and moe.router.expert_bias.abs().max() > 0
+    # the router may read another tensor than the experts do
+    route_on = torch.randn(200, 256, device=DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert not torch.equal(moe(x, route_on=route_on), moe(x))
+    # the per-expert loop is the eager test arm: the swap refuses it and says why
+    loop = MoEMLP(256, hidden=128, num_experts=4, top_k=2, num_shared=0, dense_fallback=True).to(DEV)
+    rep = swap_mxfp8(loop)
+    assert rep.blocking and any("dense_fallback" in why for _, why in rep.skipped)

@@ -67,10 +67,10 @@ def test_refresh_mxfp8_weights_serves_all_modules_at_once():
             super().__init__()
             self.proj = torch.nn.ModuleList(MXFP8Linear(256, n) for n in (256, 384, 100, 1024))  # 100: padded out_features
             self.ffn = MXFP8SwiGLU(256, hidden=512)
-            self.moe = MoEMLP(256, 128, 8, 2)
-            self.moe_small = MoEMLP(256, 96, 4, 2)  # 2H = 192 rows per expert: not one matrix, refreshes alone
+            self.moe = MoEMLP(256, hidden=128, num_experts=8, top_k=2, num_shared=0)
+            self.moe_small = MoEMLP(256, hidden=96, num_experts=4, top_k=2, num_shared=0)  # 2H = 192 rows per expert: not one matrix, refreshes alone
 
-    model = Block().to(DEV)
+    model = Block().to(DEV, torch.bfloat16)
     swap_mxfp8(model)
     model.ffn.enable_mxfp8()
 

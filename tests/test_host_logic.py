@@ -97,7 +97,7 @@ def test_swap_accounting_on_cpu():
     assert report.mac["fp8"] == 128 * 128 + 2 * 128 * 64 + 128 * 128 + 3 * 128 * 256 + 64
     assert report.mac["skipped"] == 3 * 128 * 128 + 64 and report.mac["unreached"] == 64 and report.mac["never"] == 96
     assert abs(sum(report.share(b) for b in ("fp8", "skipped", "unreached", "never")) - 1.0) < 1e-9
-    assert "SKIPPED biased.w_in" in report.summary() and "UNACCOUNTED" in report.summary()
+    assert "[skipped] biased.w_in: has a bias" in report.summary() and "[unaccounted] stray(3, 3)" in report.summary()
     # 6 swapped linears + the declaring module that converted
     assert refresh_mxfp8_weights(model) == 7 and model.mlp.w_in.refreshed == 1
     # scope: everything outside is reported, left alone, and does not block
@@ -171,3 +171,45 @@ def test_oracle_gemm_matches_scalar_and_grouped_loop(oracle):
     dw = oracle.grouped_wgrad(a, a, offsets)
     assert dw.shape == (3, 96, 96) and (dw[1] == 0).all()
     assert torch.allclose(dw[0], a[:5].double().T @ a[:5].double())
+
+
+def test_moe_block_builds_from_a_reference_spec():
+    """``build({"name": "moe", ...}, MLP, dim=...)`` with the reference's keywords; ``swap_mxfp8`` converts the result.
+
+    Nothing here runs a kernel: building, declaring and converting are host logic.
+    """
+    from kohakuwullm_amd.models.mlp import GLUMLP
+    from kohakuwullm_amd.models.moe import MoEMLP, TopKRouter
+    from kohakuwullm_amd.models.mxfp8_swap import swap_mxfp8
+    from kohakuwullm_amd.registry import MLP, ROUTER, build
+
+    assert "moe" in MLP and "swiglu" in MLP and "topk" in ROUTER
+    spec = {"name": "moe", "hidden": 512, "num_experts": 64, "top_k": 6, "num_shared": 0}
+    moe = build(spec, MLP, dim=1024)
+    assert isinstance(moe, MoEMLP) and isinstance(moe.router, TopKRouter)
+    assert moe.w_in.shape == (64, 1024, 1024) and moe.w_out.shape == (64, 1024, 512) and moe.shared is None
+    assert moe.router.weight.shape == (64, 1024) and moe.router.top_k == 6 and moe.num_buckets == 64
+    report = swap_mxfp8(moe, linear_cls=_StubLinear)
+    assert not report.blocking and sorted(report.swapped) == ["w_in", "w_out"] and report.modules == [""]
+    assert moe._routed == moe._routed_mxfp8 and callable(moe.refresh_quantized_weight)
+    assert report.mac["fp8"] == 6 * 3 * 512 * 1024 and report.mac["never"] == 64 * 1024
+
+    # every keyword of the reference's constructor, a router given as a spec with its own keywords
+    full = build({"name": "moe", "ratio": 2.0, "multiple_of": 64, "num_experts": 8, "top_k": 2, "num_shared": 2, "bias": False,
+                  "router": {"name": "topk", "score_func": "softmax"}, "router_dim": 96, "dense_fallback": False,
+                  "expert_path": "eager", "n_groups": 2, "topk_groups": 1, "bias_update_rate": 0.0}, MLP, dim=256)
+    assert full.hidden == 384 and isinstance(full.shared, GLUMLP) and full.shared.hidden == 768
+    assert full.router.weight.shape == (8, 96) and full.router.n_groups == 2 and full.router.expert_bias is None
+    assert full.expert_path == "eager" and not full.emits_router_loss and full.router_losses() is None
+    idx, weight, counts = full.router.route(torch.randn(50, 96))
+    assert idx.shape == (50, 2) and int(counts.sum()) == 100
+    assert torch.allclose(weight.sum(-1), torch.ones(50), atol=1e-5)
+    assert ((idx[:, 0] // 4) == (idx[:, 1] // 4)).all()  # one group of four experts per token
+    report = swap_mxfp8(full, linear_cls=_StubLinear)
+    assert not report.blocking and {"w_in", "w_out", "shared.w_in", "shared.w_out"} == set(report.swapped)
+    with pytest.raises(ValueError, match="expert_path"):
+        build({"name": "moe", "expert_path": "triton"}, MLP, dim=128)
+    with pytest.raises(ValueError, match="score_func"):
+        build({"name": "moe", "score_func": "relu"}, MLP, dim=128)
+    loop = build({"name": "moe", "hidden": 128, "num_experts": 4, "top_k": 2, "dense_fallback": True}, MLP, dim=128)
+    assert "dense_fallback" in loop.mxfp8_matmul()["w_in"].refusal
