@@ -88,8 +88,34 @@ def zipf_counts(num_experts: int = 64, total: int = 98304, cap: int = 16384, s: 
     return [int(v) for v in c]
 
 
-def make_moe_inputs(tokens: int = 16384, dim: int = 1024, hidden: int = 512, num_experts: int = 64, top_k: int = 6):
-    """BASELINE configs[3]: routed experts with Zipf(1.1) loads; sorted position m -> token m mod T, slot m div T."""
+def ranked_counts(num_experts: int = 64, total: int = 98304, cap: int = 16384, s: float = 1.1, empty: int = 5):
+    """Zipf(s) loads by rank instead of by draw: expert of rank r gets ~ r^-s of the rows (capped), `empty` experts none.
+
+    The seeded draws of `zipf_counts` happen to give six full experts and 58 empty ones; this routing keeps
+    59 experts alive with loads from 16384 rows down to a few dozen, so ragged tiles are what gets measured.
+    """
+    import torch
+
+    live = num_experts - empty
+    p = torch.arange(1, live + 1, dtype=torch.float64) ** -s
+    c = torch.floor(p / p.sum() * total).long().clamp(max=cap)
+    i = 0
+    while int(c.sum()) < total:
+        add = min(cap - int(c[i]), total - int(c.sum()))
+        c[i] += add
+        i += 1
+    perm = torch.randperm(num_experts, generator=torch.Generator().manual_seed(SEED))
+    out = torch.zeros(num_experts, dtype=torch.long)
+    out[perm[:live]] = c
+    return out.tolist()
+
+
+def make_moe_inputs(tokens: int = 16384, dim: int = 1024, hidden: int = 512, num_experts: int = 64, top_k: int = 6,
+                    routing: str = "draws"):
+    """BASELINE configs[3]: routed experts with Zipf(1.1) loads; sorted position m -> token m mod T, slot m div T.
+
+    routing "draws": per-expert loads drawn i.i.d. Zipf as the configuration says; "ranked": `ranked_counts`.
+    """
     import torch
 
     g = torch.Generator().manual_seed(SEED)
@@ -98,7 +124,7 @@ def make_moe_inputs(tokens: int = 16384, dim: int = 1024, hidden: int = 512, num
     w_out = (torch.randn(num_experts, dim, hidden, generator=g) * 0.02).bfloat16()
     gate = (torch.rand(tokens * top_k, generator=g) * 0.5 + 0.5).bfloat16()
     dout = (torch.randn(tokens, dim, generator=g) * 1e-2).bfloat16()
-    counts = zipf_counts(num_experts, tokens * top_k, tokens)
+    counts = (zipf_counts if routing == "draws" else ranked_counts)(num_experts, tokens * top_k, tokens)
     offsets = torch.zeros(num_experts + 1, dtype=torch.int32)
     offsets[1:] = torch.tensor(counts).cumsum(0)
     m = torch.arange(tokens * top_k)
@@ -138,14 +164,17 @@ def make_outlier_inputs(n: int = 8192):
     return x, w, dy, special
 
 
-def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
-    """The oracle's formulas with PyTorch CPU ops on the first `sample_tokens` tokens."""
+def cpu_baseline(sample_tokens: int = TOKENS, device_rows=None) -> dict:
+    """The oracle's formulas with PyTorch CPU ops on the first `sample_tokens` tokens.
+
+    `device_rows` = (row indices, the device's output rows for them): the same leg, being the checker, also states
+    how far the measured path's forward output is from the oracle's chain on those rows (relative Frobenius error)."""
     import torch
 
     from oracle import mx_oracle as ora
 
-    x, w_in, w_out, dy = make_inputs(TOKENS)
-    x, dy = x[:sample_tokens].contiguous(), dy[:sample_tokens].contiguous()
+    x_all, w_in, w_out, dy = make_inputs(TOKENS)
+    x, dy = x_all[:sample_tokens].contiguous(), dy[:sample_tokens].contiguous()
     f32 = torch.float32
 
     def q_rows(t):
@@ -179,7 +208,16 @@ def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
         one_step()
         steps += 1
     dt_step = (time.perf_counter() - t0) / steps
+    accuracy = {}
+    if device_rows is not None:
+        rows, y_dev = device_rows
+        gu = ora.gemm_nt(*ora.quantize_rows(x_all[rows]), *win_f).bfloat16().float()
+        g, u = gu.chunk(2, dim=-1)
+        y_ref = ora.gemm_nt(*ora.quantize_rows(g * torch.sigmoid(g) * u), *wout_f)
+        accuracy = {"rel_error": float(f"{ora.rel_error(y_dev, y_ref):.3e}"),
+                    "rel_error_of": f"forward output of {len(rows)} sampled tokens against the oracle's dequantize-then-matmul chain in fp64"}
     return {
+        **accuracy,
         "value": step_flops(sample_tokens) / dt_step / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
@@ -190,16 +228,96 @@ def cpu_baseline(sample_tokens: int = TOKENS) -> dict:
     }
 
 
+
+def _event_times(fn, iters: int, warm: int = 3):
+    """Device times (ms) of `iters` calls of fn, each bracketed by events on the current stream."""
+    import torch
+
+    for _ in range(warm):
+        fn()
+    pairs = []
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) for a, b in pairs)
+
+
+def measure_stream(dev, out_bytes: int = 1 << 30, iters: int = 10) -> dict:
+    """Streaming bandwidth of this device in GB/s (best and median of `iters` launches on 1 GiB per operand):
+    read, copy, triad, and a 2-bytes-read-per-byte-written mix (the traffic of a 16-bit -> 8-bit cast)."""
+    import torch
+
+    from kohakuwullm_amd import _lib
+
+    lib = _lib.load()
+    a = torch.empty(2 * out_bytes, dtype=torch.uint8, device=dev).random_(0, 255)  # kind 3 reads twice what it writes
+    b = torch.empty(out_bytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    c = torch.empty(out_bytes, dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream(dev).cuda_stream
+    out = {}
+    for name, kind, moved in (("read", 0, out_bytes), ("copy", 1, 2 * out_bytes), ("triad", 2, 3 * out_bytes), ("read2_write1", 3, 3 * out_bytes)):
+        ts = _event_times(lambda: _lib.check(lib.mx_ubench_stream(kind, a.data_ptr(), b.data_ptr(), c.data_ptr(), out_bytes, st),
+                                             "mx_ubench_stream"), iters)
+        out[name] = {"best": round(moved / ts[0] / 1e6, 1), "median": round(moved / ts[len(ts) // 2] / 1e6, 1)}
+    del a, b, c
+    return out
+
+
+def measure_mfma(dev, iters: int = 4000, repeats: int = 5) -> dict:
+    """Issue rate of the block-scaled fp8 MFMA from registers in TFLOP/s: both tile shapes, zero and hashed operands."""
+    import torch
+
+    from kohakuwullm_amd import _lib
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.empty(cus * 512, dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream(dev).cuda_stream
+    out = {}
+    for wide, shape, flop in ((0, "16x16x128", 2.0 * 16 * 16 * 128), (1, "32x32x64", 2.0 * 32 * 32 * 64)):
+        for random, label in ((1, "hashed"), (0, "zeros")):
+            count = []
+
+            def launch():
+                n = lib.mx_ubench_mfma(wide, iters, random, sink.data_ptr(), sink.numel(), st)
+                if n < 0:
+                    _lib.check(int(n), "mx_ubench_mfma")
+                count.append(n)
+
+            ts = _event_times(launch, repeats)
+            out[f"{shape}_{label}"] = {"best": round(count[0] * flop / ts[0] / 1e9, 1),
+                                       "median": round(count[0] * flop / ts[len(ts) // 2] / 1e9, 1)}
+    return out
+
+
+def measured_peaks(dev) -> dict:
+    """The two denominators measured on this device, beside the nominal ones: the best streaming pattern (GB/s) and the
+    MFMA loop on hashed operands (TFLOP/s; zero operands clock higher and are reported by --workload peak)."""
+    stream, mfma = measure_stream(dev, iters=5), measure_mfma(dev, iters=2000, repeats=3)
+    return {
+        "hbm_gbs": max(v["best"] for v in stream.values()),
+        "hbm_read2_write1_gbs": stream["read2_write1"]["best"],
+        "hbm_copy_gbs": stream["copy"]["best"],
+        "mfma_tflops": max(v["best"] for k, v in mfma.items() if k.endswith("hashed")),
+        "how": "mx_ubench_stream on 1 GiB per operand, mx_ubench_mfma from registers; best of a few launches, this run",
+    }
+
 # Bytes the GEMM launches of one step move between the L2s and the fabric, per launch, from the
 # FETCH_SIZE and WRITE_SIZE counter runs summarised under profiles/ (each scaled by what the
 # counter reads for a device copy of known size): 2084 MiB over 4 launches.
 GEMM_TRAFFIC_PER_LAUNCH = {"ffn": 521 * 2**20}
+TRAFFIC_SOURCE = ("a constant, not measured in this run: the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in "
+                  "profiles/gemm_nt_kernel_dense_ffn_fwd_bwd.md")
 
 GEMM_ENTRIES = ("mx_gemm_nt", "mx_gemm_nt_batch", "mx_grouped_gemm_nt", "mx_experts_gemm1", "mx_experts_scatter_gemm",
                 "mx_experts_gemm2_dgrad", "mx_grouped_wgrad_nt")
 
 
-def build_workload(name: str, dev):
+def build_workload(name: str, dev, routing: str = "draws"):
     """Returns (step(i), gflop per step, description, refresh())."""
     import torch
 
@@ -226,6 +344,14 @@ def build_workload(name: str, dev):
             mxfp8_swiglu_mlp(x, w_in, w_out, state["packed"]).backward(dys[i % ncopies])
             x.grad = w_in.grad = w_out.grad = None
 
+        def sample_rows(n=64):
+            """(row indices, the measured path's forward output on those rows) for the accuracy figure."""
+            rows = torch.randperm(TOKENS, generator=torch.Generator().manual_seed(SEED))[:n]
+            with torch.no_grad():
+                y = mxfp8_swiglu_mlp(xs[0].detach(), w_in.detach(), w_out.detach(), state["packed"])
+            return rows, y[rows.to(dev)].cpu()
+
+        step.sample_rows = sample_rows
         desc = "dense 546M-class SwiGLU FFN fwd+bwd: tokens 16384, dim 1536, ffn 4096 (BASELINE configs[1])"
         return step, step_flops(TOKENS) / 1e9, desc, refresh
     if name == "attn":
@@ -254,7 +380,7 @@ def build_workload(name: str, dev):
         gflop = 3 * (2.0 * t * w_qkv_h.shape[0] * d + 2.0 * t * d * d) / 1e9
         return step, gflop, "GQA attention projections fwd+dgrad+wgrad: tokens 32768, dim 2048, W_qkv 3072x2048, W_o 2048x2048 (BASELINE configs[2])", refresh
     if name == "moe":
-        x_h, w_in_h, w_out_h, gate_h, dout_h, offsets, order, token_of, counts = make_moe_inputs()
+        x_h, w_in_h, w_out_h, gate_h, dout_h, offsets, order, token_of, counts = make_moe_inputs(routing=routing)
         xs = [x_h.to(dev).requires_grad_(True) for _ in range(ncopies)]
         w_in, w_out = w_in_h.to(dev).requires_grad_(True), w_out_h.to(dev).requires_grad_(True)
         gate = gate_h.to(dev).requires_grad_(True)
@@ -270,7 +396,10 @@ def build_workload(name: str, dev):
             x.grad = w_in.grad = w_out.grad = gate.grad = None
 
         m, dim, hid = int(sum(counts)), x_h.shape[1], w_out_h.shape[2]
-        return step, 3 * 6.0 * m * dim * hid / 1e9, "routed experts fwd+bwd: 64 experts (Zipf 1.1 loads, 58 empty), top-6, tokens 16384, dim 1024, hidden 512 (BASELINE configs[3])", refresh
+        live = sum(1 for c in counts if c)
+        how = "Zipf 1.1 draws" if routing == "draws" else "Zipf 1.1 by rank"
+        return step, 3 * 6.0 * m * dim * hid / 1e9, (f"routed experts fwd+bwd: 64 experts ({how}: {live} with rows, {64 - live} empty, largest "
+                                                     f"{max(counts)} rows), top-6, tokens 16384, dim 1024, hidden 512 (BASELINE configs[3])"), refresh
     if name == "outlier":
         x_h, w_h, dy_h, _ = make_outlier_inputs()
         x, w, dy = x_h.to(dev), w_h.to(dev), dy_h.to(dev)
@@ -385,13 +514,92 @@ STREAM_METRICS = {
 }
 
 
+QUANT_SHAPES = ((16384, 1536), (16384, 4096), (32768, 2048), (8192, 8192))  # activations of BASELINE configs[1], [1], [2], [4]
+
+
+def run_quant(dev, iters: int) -> dict:
+    """The stand-alone quantizers (rows, columns, both) on the activation shapes, cold: every launch reads a copy of
+    the input that left the 256 MB last-level cache several launches ago.  Per kernel and shape: algorithmic bytes
+    (3.03125 B/element for one axis, 4.0625 for both) / device time from events around each launch."""
+    import torch
+
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx, quantize_mx_cols, quantize_mx_dual
+
+    g = torch.Generator().manual_seed(SEED)
+    rows_out, total_bytes, total_ms = [], 0.0, 0.0
+    for m, k in QUANT_SHAPES:
+        copies = max(3, -(-(768 << 20) // (m * k * 2)))  # at least 768 MB of distinct inputs in rotation
+        base = torch.randn(m, k, generator=g).bfloat16()
+        xs = [base.to(dev).add_(0) for _ in range(copies)]
+        for name, fn, per_elem in (("rows", quantize_mx, 3.03125), ("cols", quantize_mx_cols, 3.03125),
+                                   ("dual", quantize_mx_dual, 4.0625)):
+            state = {"i": 0}
+
+            def call():
+                fn(xs[state["i"] % copies])
+                state["i"] += 1
+
+            ts = _event_times(call, iters, warm=copies)
+            nbytes = m * k * per_elem
+            med, best = ts[len(ts) // 2], ts[0]
+            rows_out.append({"kernel": f"quantize_mx_{name}", "shape": [m, k], "us_median": round(med * 1e3, 2),
+                             "us_best": round(best * 1e3, 2), "gbs_median": round(nbytes / med / 1e6, 1),
+                             "gbs_best": round(nbytes / best / 1e6, 1)})
+            total_bytes += nbytes * len(ts)
+            total_ms += sum(ts)
+        del xs
+    return {"kernels": rows_out, "gbs": total_bytes / total_ms / 1e6, "launches": len(rows_out) * iters,
+            "avg_us": total_ms / (len(rows_out) * iters) * 1e3}
+
+
+def standalone_line(args, dev) -> dict:
+    """--workload stream | peak | quant: one JSON line each, the same schema as the step workloads."""
+    common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None, "data": "synthetic"}
+    if args.workload == "stream":
+        bw = measure_stream(dev, iters=max(args.steps, 10))
+        best = max(v["best"] for v in bw.values())
+        return {"metric": "device streaming bandwidth GB/s (best of read / copy / triad / 2:1 mix)", "value": best, "unit": "GB/s",
+                "ms_per_step": None, "dtype": "bytes", **common,
+                "config": {"workload": "1 GiB per operand, non-temporal 16-byte accesses, grid-stride (mx_ubench_stream)", "patterns": bw},
+                "roofline": {"kernel": "stream_kernel", "bound": "hbm", "achieved": best, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(best / HBM_PEAK_GBS, 4), "traffic": None}}
+    if args.workload == "peak":
+        mf = measure_mfma(dev, repeats=max(args.steps // 4, 5))
+        best = max(v["best"] for k, v in mf.items() if k.endswith("hashed"))
+        return {"metric": "block-scaled fp8 MFMA issue rate from registers TFLOP/s (hashed operands)", "value": best, "unit": "TFLOP/s",
+                "ms_per_step": None, "dtype": "e4m3 x e4m3, ue8m0 scales, fp32 accumulate", **common,
+                "config": {"workload": "8 waves per CU, 8 (16x16x128) or 4 (32x32x64) independent accumulator tiles per wave, "
+                                       "4000 rounds, no memory traffic (mx_ubench_mfma)", "variants": mf},
+                "roofline": {"kernel": "mfma_peak_kernel", "bound": "mfma", "achieved": best, "peak": MFMA_PEAK_TFLOPS,
+                             "unit": "TFLOP/s", "frac": round(best / MFMA_PEAK_TFLOPS, 4), "traffic": None}}
+    q = run_quant(dev, max(args.steps, 20))
+    peaks = measured_peaks(dev)
+    return {"metric": "MXFP8 quantizer GB/s (rows, columns, both; activation shapes, cold inputs)", "value": round(q["gbs"], 1),
+            "unit": "GB/s", "ms_per_step": None, "dtype": "bf16 -> e4m3 + ue8m0", **common,
+            "config": {"workload": "quantize_mx / quantize_mx_cols / quantize_mx_dual on 16384x1536, 16384x4096, 32768x2048, "
+                                   "8192x8192 bf16; inputs rotate through >= 768 MB of copies", "kernels": q["kernels"]},
+            "roofline": {"kernel": "quant_rows_kernel, quant_cols_kernel<false>, quant_cols_kernel<true>", "bound": "hbm",
+                         "achieved": round(q["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(q["gbs"] / HBM_PEAK_GBS, 4),
+                         "traffic": None, "launches": q["launches"], "avg_launch_us": round(q["avg_us"], 2),
+                         "peak_measured": peaks["hbm_gbs"], "frac_of_measured": round(q["gbs"] / peaks["hbm_gbs"], 4),
+                         "peak_measured_read2_write1": peaks["hbm_read2_write1_gbs"]}}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="ffn", choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh", "heads"),
-                    help="ffn (default) is the configuration the headline metric is quoted on")
+    ap.add_argument("--workload", default="ffn",
+                    choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh", "heads", "quant", "stream", "peak"),
+                    help="ffn (default) is the configuration the headline metric is quoted on; quant: the stand-alone "
+                         "quantizers; stream / peak: the device's measured bandwidth and MFMA rate")
+    ap.add_argument("--routing", default="draws", choices=("draws", "ranked"),
+                    help="moe: per-expert loads drawn i.i.d. Zipf (six full experts with the fixed seed) or Zipf by rank (59 live experts)")
+    ap.add_argument("--samples", type=int, default=0,
+                    help="after the timed region, time this many further steps one by one (events around each) and report "
+                         "their median and best; 100 or more for a publishable distribution")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -407,7 +615,10 @@ def main() -> None:
 
     dev = torch.device("cuda:0")
     _lib.check(_lib.load().mx_device_supported(0), "mx_device_supported")
-    step, gflop, desc, refresh = build_workload(args.workload, dev)
+    if args.workload in ("quant", "stream", "peak"):
+        print(json.dumps(standalone_line(args, dev)))
+        return
+    step, gflop, desc, refresh = build_workload(args.workload, dev, args.routing)
 
     refresh()
     torch.cuda.synchronize()
@@ -427,6 +638,17 @@ def main() -> None:
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     tflops = gflop / ms_per_step
+
+    sampled = {}
+    if args.samples > 0:
+        counter = {"i": 0}
+
+        def one():
+            step(counter["i"])
+            counter["i"] += 1
+
+        ts = _event_times(one, args.samples, warm=0)
+        sampled = {"ms_per_step_median": round(ts[len(ts) // 2], 4), "ms_per_step_best": round(ts[0], 4), "samples": len(ts)}
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -457,6 +679,7 @@ def main() -> None:
     if not gemm:
         # a workload of streaming kernels only: the figure of merit is bytes per second against HBM
         step_bytes = quant_bytes / args.steps
+        stream_peak = max(v["best"] for v in measure_stream(dev, iters=5).values())
         extra = {}
         if hasattr(step, "alternative"):  # the same work done another way, timed the same way, for comparison
             key, other = step.alternative
@@ -475,11 +698,13 @@ def main() -> None:
             "data": "synthetic", "config": {"workload": desc, "bytes_per_step": int(step_bytes)},
             "roofline": {"kernel": ", ".join(sorted({n for n, _, _ in quant})), "bound": "hbm", "achieved": round(quant_gbs, 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "peak_measured": stream_peak, "frac_of_measured": round(quant_gbs / stream_peak, 4),
                          "launches": len(quant), "avg_launch_us": round(quant_ms / len(quant) * 1e3, 2)},
-            **extra,
+            **sampled, **extra,
         }))
         return
     gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    peaks = measured_peaks(dev)
 
     out = {
         "metric": "MXFP8 linear fwd+bwd TFLOP/s (quantizers included)",
@@ -489,6 +714,7 @@ def main() -> None:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
+        **sampled,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -508,6 +734,9 @@ def main() -> None:
             "unit": "TFLOP/s",
             "frac": round(gemm_tflops / MFMA_PEAK_TFLOPS, 4),
             "traffic": GEMM_TRAFFIC_PER_LAUNCH.get(args.workload),
+            "traffic_source": TRAFFIC_SOURCE if args.workload in GEMM_TRAFFIC_PER_LAUNCH else None,
+            "peak_measured": peaks["mfma_tflops"],
+            "frac_of_measured": round(gemm_tflops / peaks["mfma_tflops"], 4),
             "launches": len(gemm),
             "avg_launch_us": round(gemm_ms / len(gemm) * 1e3, 2),
             "gflop_per_launch": round(gemm_flops / len(gemm) / 1e9, 2),
@@ -519,14 +748,17 @@ def main() -> None:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(quant_gbs / HBM_PEAK_GBS, 4),
+            "peak_measured": peaks["hbm_gbs"],
+            "frac_of_measured": round(quant_gbs / peaks["hbm_gbs"], 4),
             "launches": len(quant),
             "avg_launch_us": round(quant_ms / len(quant) * 1e3, 2),
             "share_of_step": round(quant_ms / (quant_ms + gemm_ms), 4),
         },
+        "peaks_measured": peaks,
         "weight_refresh_ms": round(weight_refresh_ms, 4),
     }
     if not args.no_cpu_baseline and args.workload == "ffn":
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(device_rows=step.sample_rows())
     print(json.dumps(out))
 
 

@@ -203,29 +203,8 @@ def test_attention_projections_sampled_oracle(oracle, attn):
 # ----------------------------------------------------------------------------- routed experts
 
 
-def _ranked_counts(num_experts=64, total=98304, cap=16384, s=1.1, empty=5):
-    """Deterministic Zipf-by-rank loads: every tile-boundary case at once, `empty` experts with no tokens."""
-    live = num_experts - empty
-    p = torch.arange(1, live + 1, dtype=torch.float64) ** -s
-    c = torch.floor(p / p.sum() * total).long().clamp(max=cap)
-    i = 0
-    while int(c.sum()) < total:
-        add = min(cap - int(c[i]), total - int(c.sum()))
-        c[i] += add
-        i += 1
-    perm = torch.randperm(num_experts, generator=torch.Generator().manual_seed(SEED))
-    out = torch.zeros(num_experts, dtype=torch.long)
-    out[perm[:live]] = c
-    return out.tolist()
-
-
 def _moe_problem(kind):
-    x, w_in, w_out, gate, dout, offsets, order, token_of, counts = bench.make_moe_inputs()
-    if kind == "ranked":
-        counts = _ranked_counts()
-        offsets = torch.zeros(len(counts) + 1, dtype=torch.int32)
-        offsets[1:] = torch.tensor(counts).cumsum(0)
-    return x, w_in, w_out, gate, dout, offsets, order, token_of, counts
+    return bench.make_moe_inputs(routing="ranked" if kind == "ranked" else "draws")
 
 
 @pytest.mark.parametrize("kind", ["zipf_draws", "ranked"])
