@@ -40,7 +40,8 @@ enum mx_status {
     MX_EUNSUPPORTED = -2, /* well-formed request this build has no kernel for */
     MX_ELAUNCH = -3,     /* the HIP runtime refused the launch */
     MX_ENODEV = -4,      /* the current device is not gfx950 */
-    MX_ECAPTURE = -5     /* the stream is being captured into a graph: nothing was launched */
+    MX_ECAPTURE = -5,    /* the stream is being captured into a graph: nothing was launched */
+    MX_ETOOBIG = -6      /* the request exceeds the fixed capacity of an entry point that allocates nothing */
 };
 
 enum mx_dtype { MX_BF16 = 0, MX_FP16 = 1, MX_FP32 = 2 };
@@ -410,6 +411,23 @@ int64_t mx_expert_sort_workspace(int64_t n, int64_t num_buckets);
 int mx_expert_sort(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
                    int64_t num_buckets, int32_t *offsets, int32_t *order, int32_t *token_of, int32_t *max_rows,
                    int32_t *workspace, int64_t workspace_len, void *stream);
+
+/*
+ * mx_expert_sort for callers that can bring no workspace and must not allocate one: a tight serving loop
+ * whose buffers were sized once, a harness that forbids hipMalloc.  It has no counterpart in the reference
+ * (there, torch allocates inside expert_sort).  Same arguments without the workspace, same results bit for
+ * bit; the scratch is a fixed array of MX_EXPERT_SORT_STATIC_WORDS int32 (4 MiB) inside the library's code
+ * object, resident on every GPU the library is used on until the process ends.  The call performs no
+ * hipMalloc / hipFree and no allocating library call.  A request that needs more than the array holds
+ * (mx_expert_sort_workspace(n, num_buckets) > MX_EXPERT_SORT_STATIC_WORDS; never the case for
+ * num_buckets <= 256) returns MX_ETOOBIG and launches nothing.  All calls on one GPU share that GPU's
+ * array: calls that may overlap in time on one GPU (different streams, different threads) race and must be
+ * serialised by the caller; calls in one stream are safe.
+ */
+#define MX_EXPERT_SORT_STATIC_WORDS (1 << 20)
+int mx_expert_sort_static(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
+                          int64_t num_buckets, int32_t *offsets, int32_t *order, int32_t *token_of, int32_t *max_rows,
+                          void *stream);
 
 /*
  * out (num_tokens, d)[t] = sum over the sorted positions p < valid_rows[0] with

@@ -17,7 +17,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmxfp8_hip.so")
 
-MX_OK, MX_EINVAL, MX_EUNSUPPORTED, MX_ELAUNCH, MX_ENODEV, MX_ECAPTURE = 0, -1, -2, -3, -4, -5
+MX_OK, MX_EINVAL, MX_EUNSUPPORTED, MX_ELAUNCH, MX_ENODEV, MX_ECAPTURE, MX_ETOOBIG = 0, -1, -2, -3, -4, -5, -6
 MX_ABI_VERSION = 2
 MX_DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
@@ -60,6 +60,7 @@ SIGNATURES = {
     "mx_expert_counts": (_ci, [_p, _ci, _i64, _i64, _p, _p]),
     "mx_expert_sort_workspace": (_i64, [_i64, _i64]),
     "mx_expert_sort": (_ci, [_p, _ci, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _p]),
+    "mx_expert_sort_static": (_ci, [_p, _ci, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p]),
     "mx_combine_routed": (_ci, [_p, _ci, _i64, _p, _ci, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p]),
     "mx_combine_routed_backward": (
         _ci, [_p, _i64, _p, _i64, _ci, _p, _ci, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _p, _p]),

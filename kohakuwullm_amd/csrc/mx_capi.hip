@@ -14,6 +14,9 @@ extern "C" const char *mx_strerror(int status) {
     case MX_ENODEV: return "the device is not a gfx950 (MI355X-class) GPU";
     case MX_ECAPTURE:
         return "the stream is being captured into a graph: this library refuses to be recorded (run it eagerly)";
+    case MX_ETOOBIG:
+        return "the request needs more scratch than the fixed array of this no-allocation entry point holds; use the "
+               "variant that takes a caller workspace";
     default: return "unknown status";
     }
 }

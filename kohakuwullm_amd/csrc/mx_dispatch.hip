@@ -14,6 +14,8 @@
 //
 // All of it is index and byte traffic: the combine streams top_k rows per token at HBM rate,
 // the sort moves 12 bytes per pair.
+#include <atomic>
+
 #include "mx_common.h"
 
 namespace mx {
@@ -414,21 +416,17 @@ extern "C" int64_t mx_expert_sort_workspace(int64_t n, int64_t num_buckets) {
     return chunks * num_buckets;
 }
 
-extern "C" int mx_expert_sort(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
-                              int64_t num_buckets, int32_t *offsets, int32_t *order, int32_t *token_of,
-                              int32_t *max_rows, int32_t *workspace, int64_t workspace_len, void *stream) {
-    if (n < 0 || n >= 0x7FFFFFFF || num_buckets <= 0 || top_k <= 0 || (idx_bytes != 4 && idx_bytes != 8) || !counts ||
-        !offsets || (n > 0 && (!flat_expert || !order || !token_of)))
-        return MX_EINVAL;
-    if (num_buckets > MAX_SORT_BUCKETS) return MX_EUNSUPPORTED;
-    const int64_t need = mx_expert_sort_workspace(n, num_buckets);
-    if (!workspace || workspace_len < need) return MX_EINVAL;
-    hipStream_t st = (hipStream_t)stream;
-    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
+// The three launches of the sort on a workspace of `need` = chunks * num_buckets words that the caller of this
+// function vouches for (the public entry points check where it comes from and how large it is).
+static int sort_launch(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
+                       int64_t num_buckets, int32_t *offsets, int32_t *order, int32_t *token_of, int32_t *max_rows,
+                       int32_t *workspace, int64_t need, hipStream_t st) {
     const int rounds = sort_rounds(n), buckets = (int)num_buckets;
     const int chunks = (int)(need / num_buckets);
     const size_t lds = (size_t)buckets * sizeof(int32_t);
     const dim3 wave(64);
+    // every word of workspace[0, need) is written before it is read: by the fill when there are no pairs, else by
+    // the histogram pass (each chunk writes its count for every bucket), so nothing of an earlier call survives
     if (n == 0) dispatch_fill_kernel<<<dim3((unsigned)((need + 255) / 256)), dim3(256), 0, st>>>(workspace, need, 0);
     if (n && idx_bytes == 8) sort_hist_kernel<true><<<dim3((unsigned)chunks), wave, lds, st>>>(flat_expert, n, buckets, rounds, chunks, workspace);
     if (n && idx_bytes == 4) sort_hist_kernel<false><<<dim3((unsigned)chunks), wave, lds, st>>>(flat_expert, n, buckets, rounds, chunks, workspace);
@@ -436,6 +434,61 @@ extern "C" int mx_expert_sort(const void *flat_expert, int idx_bytes, int64_t n,
     if (n && idx_bytes == 8) sort_place_kernel<true><<<dim3((unsigned)chunks), wave, lds, st>>>(flat_expert, n, buckets, rounds, chunks, (int)top_k, workspace, order, token_of);
     if (n && idx_bytes == 4) sort_place_kernel<false><<<dim3((unsigned)chunks), wave, lds, st>>>(flat_expert, n, buckets, rounds, chunks, (int)top_k, workspace, order, token_of);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+static int sort_args_ok(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
+                        int64_t num_buckets, const int32_t *offsets, const int32_t *order, const int32_t *token_of) {
+    if (n < 0 || n >= 0x7FFFFFFF || num_buckets <= 0 || top_k <= 0 || (idx_bytes != 4 && idx_bytes != 8) || !counts ||
+        !offsets || (n > 0 && (!flat_expert || !order || !token_of)))
+        return MX_EINVAL;
+    return num_buckets > MAX_SORT_BUCKETS ? MX_EUNSUPPORTED : MX_OK;
+}
+
+extern "C" int mx_expert_sort(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts, int64_t top_k,
+                              int64_t num_buckets, int32_t *offsets, int32_t *order, int32_t *token_of,
+                              int32_t *max_rows, int32_t *workspace, int64_t workspace_len, void *stream) {
+    const int rc = sort_args_ok(flat_expert, idx_bytes, n, counts, top_k, num_buckets, offsets, order, token_of);
+    if (rc != MX_OK) return rc;
+    const int64_t need = mx_expert_sort_workspace(n, num_buckets);
+    if (!workspace || workspace_len < need) return MX_EINVAL;
+    hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
+    return sort_launch(flat_expert, idx_bytes, n, counts, top_k, num_buckets, offsets, order, token_of, max_rows, workspace,
+                       need, st);
+}
+
+// Scratch of mx_expert_sort_static: a fixed array in the code object, so the entry point has nothing to allocate.
+// Every device the library runs on holds its own copy at its own address for the life of the process.  In host
+// code the name below is only a handle for hipGetSymbolAddress; the address kernels may use is what that call
+// returns on the device that is current, kept per device ordinal in sort_scratch_of().
+static __device__ __align__(256) int32_t scratch[MX_EXPERT_SORT_STATIC_WORDS];
+
+static int32_t *sort_scratch_of_current_device() {
+    static std::atomic<int32_t *> known[64];  // by device ordinal; written once with the only value it can hold
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    int32_t *ptr = known[dev].load(std::memory_order_acquire);
+    if (ptr) return ptr;
+    if (hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    known[dev].store(ptr, std::memory_order_release);
+    return ptr;
+}
+
+extern "C" int mx_expert_sort_static(const void *flat_expert, int idx_bytes, int64_t n, const int32_t *counts,
+                                     int64_t top_k, int64_t num_buckets, int32_t *offsets, int32_t *order,
+                                     int32_t *token_of, int32_t *max_rows, void *stream) {
+    const int rc = sort_args_ok(flat_expert, idx_bytes, n, counts, top_k, num_buckets, offsets, order, token_of);
+    if (rc != MX_OK) return rc;
+    const int64_t need = mx_expert_sort_workspace(n, num_buckets);
+    if (need > MX_EXPERT_SORT_STATIC_WORDS) return MX_ETOOBIG;
+    hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
+    int32_t *const ws = sort_scratch_of_current_device();
+    if (!ws) return MX_ELAUNCH;
+    return sort_launch(flat_expert, idx_bytes, n, counts, top_k, num_buckets, offsets, order, token_of, max_rows, ws, need, st);
 }
 
 extern "C" int mx_combine_routed(const void *rows, int dtype, int64_t ld, const void *weight, int w_dtype,

@@ -81,6 +81,30 @@ def expert_sort(flat_expert: torch.Tensor, counts: torch.Tensor, top_k: int, num
     return offsets, order, token_of, max_rows
 
 
+def expert_sort_into(flat_expert: torch.Tensor, counts: torch.Tensor, top_k: int, num_experts: int,
+                     offsets: torch.Tensor, order: torch.Tensor, token_of: torch.Tensor) -> None:
+    """:func:`expert_sort` into tensors the caller already holds, through the library entry point that allocates nothing.
+
+    For loops whose buffers were sized once and that must not allocate per call (neither here nor in the
+    library): ``offsets (E + 1,)``, ``order (n,)``, ``token_of (n,)`` int32 are overwritten; the scratch is a
+    fixed 4 MiB array inside the library (requests beyond it raise; none with 256 buckets or fewer does).
+    The results are those of :func:`expert_sort`, bit for bit.  Calls on one GPU share the scratch: issue them
+    on one stream, or serialise them.
+    """
+    flat_expert = _index_tensor(flat_expert, "flat_expert")
+    n = flat_expert.numel()
+    for t, shape, name in ((counts, (num_experts,), "counts"), (offsets, (num_experts + 1,), "offsets"), (order, (n,), "order"),
+                           (token_of, (n,), "token_of")):
+        _lib.require_gpu(t, name)
+        if t.dtype != torch.int32 or tuple(t.shape) != shape or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous int32 tensor of shape {shape}, got {t.dtype} {tuple(t.shape)}")
+    if top_k <= 0:
+        raise ValueError(f"top_k={top_k} must be positive")
+    _lib.invoke("mx_expert_sort_static", n * (flat_expert.element_size() + 8), flat_expert,
+                flat_expert.data_ptr(), _INDEX[flat_expert.dtype], n, counts.data_ptr(), top_k, num_experts,
+                offsets.data_ptr(), order.data_ptr(), token_of.data_ptr(), None)
+
+
 def _valid_ptr(valid_rows, device) -> int:
     if valid_rows is None:
         return 0
