@@ -144,6 +144,7 @@ struct ExpertTable {
     int a[MX_TABLE_MAX + 1];
     int b[MX_TABLE_MAX + 1];
     int n;
+    int longest;  // build_live_table: the K stages of the expert with the most rows
 };
 
 // a[e] = row tiles (of `bm` rows) of experts before e, b[e] = 128-row tiles of the padded token
@@ -179,11 +180,12 @@ __device__ __forceinline__ void build_live_table(ExpertTable &tb, const int32_t 
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
         const uint64_t below = lane ? ~0ull >> (64 - lane) : 0ull;
-        int carry_l = 0, carry_p = 0;
+        int carry_l = 0, carry_p = 0, most = 0;
         for (int e0 = 0; e0 < E; e0 += 64) {
             const int e = e0 + lane;
             const int rows = e < E ? offsets[e + 1] - offsets[e] : 0;
             const int pads = (rows + 127) / 128;
+            most = pads > most ? pads : most;
             const int ip = wave_incl_scan(pads, lane);
             const uint64_t mask = __ballot(rows > 0);
             if (rows > 0) {
@@ -194,9 +196,15 @@ __device__ __forceinline__ void build_live_table(ExpertTable &tb, const int32_t 
             carry_l += __builtin_popcountll(mask);
             carry_p += __shfl(ip, 63, 64);
         }
+#pragma unroll
+        for (int d = 32; d; d >>= 1) {
+            const int other = __shfl_xor(most, d, 64);
+            most = other > most ? other : most;
+        }
         if (lane == 0) {
             tb.n = carry_l;
             tb.b[carry_l] = carry_p;  // one past the last expert's K stages
+            tb.longest = most;
         }
     }
     __syncthreads();
@@ -855,7 +863,7 @@ __device__ __forceinline__ int wgrad_unit_of(int b, int g) { return (g & 7) == 0
 
 // Number of K slices per tile: as many as fill the GPU about twice over, at most 8, and 1 when
 // the tiles of the non-empty experts already fill three quarters of it.  Also counts the
-// non-empty experts.
+// non-empty experts.  (With the table, any result above 1 selects the even split.)
 __device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, int &live, const ExpertTable *tb) {
     if (tb) {
         live = tb->n;
@@ -863,8 +871,18 @@ __device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, 
         live = 0;
         for (int e = 0; e < p.E; e++) live += p.offsets[e + 1] > p.offsets[e] ? 1 : 0;
     }
-    const int tiles = live * p.tiles_m * p.tiles_n;
-    if (!p.slots || tiles == 0 || tiles * 4 >= workgroups * 3) return 1;
+    const int per_e = p.tiles_m * p.tiles_n;
+    const int tiles = live * per_e;
+    if (!p.slots || tiles == 0) return 1;
+    if (tiles * 4 >= workgroups * 3) {
+        // Plenty of tiles: dealt whole and round-robin they balance, unless a few experts hold most of the
+        // rows -- then one workgroup's tile is as long as `longest` K stages while the average workgroup has
+        // total * per_e / workgroups to do, and the launch lasts as long as that one tile.  Routed loads
+        // follow a power law, so this is the usual case: split evenly when the longest tile is more than
+        // twice the average load (the split costs each workgroup up to two fp32 partial tiles).
+        if (!tb || workgroups < per_e) return 1;
+        return (int64_t)tb->longest * workgroups > 2 * (int64_t)tb->b[tb->n] * per_e ? 2 : 1;
+    }
     int s = 2 * workgroups / tiles;
     s = s < p.slots / tiles ? s : p.slots / tiles;
     return s < 1 ? 1 : (s > 8 ? 8 : s);
