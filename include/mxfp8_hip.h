@@ -51,6 +51,9 @@ enum mx_epilogue {
     MX_EPI_NONE = 0,      /* C = A B^T, cast to c_dtype */
     MX_EPI_ACCUMULATE = 1 /* C += A B^T with fp32 atomic adds; c_dtype must be MX_FP32 */
 };
+/* OR into `epilogue` of mx_gemm_nt: run on 128 x 128 tiles with two workgroups per compute unit instead of one
+ * 256 x 256 tile (same product; a tiling choice kept selectable so the two can be timed against each other). */
+#define MX_EPI_TILE_128 0x10
 /* OR into `epilogue` to cut K into n slices that run as independent tiles (needs
  * MX_EPI_ACCUMULATE and a caller-zeroed C): fills the GPU when M*N alone gives too few tiles. */
 #define MX_EPI_SPLIT_K(n) ((n) << 8)

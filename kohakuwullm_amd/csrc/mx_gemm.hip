@@ -170,25 +170,26 @@ struct DenseProblem {
         }
         // Interior tiles of a vector-aligned C store unconditionally: every lane issues NST stores.
         const bool interior = t.m0 + S::BM <= p.M && t.n0 + S::BN <= p.N && p.c_vec && !p.accumulate;
-        // component v of a lane's 8 sub-tiles (i, 0..7): row 16 i + 4 g + v, 8 consecutive N from 8 r16
-        const int n = t.n0 + L.wn * S::WTN + 8 * L.r16;
+        // component v of a lane's NT sub-tiles (i, 0..NT-1): row 16 i + 4 g + v, NT consecutive N from NT r16
+        const int n = t.n0 + L.wn * S::WTN + S::NT * L.r16;
 #pragma unroll
         for (int i = 0; i < S::MT; i++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int m = t.m0 + L.wm * S::WTM + 16 * i + 4 * L.g + v;
                 const int64_t off = (int64_t)m * p.ldc + n;
-                const v4f lo = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
-                const v4f hi = {acc[i][4][v], acc[i][5][v], acc[i][6][v], acc[i][7][v]};
+                float run[S::NT];
+#pragma unroll
+                for (int j = 0; j < S::NT; j++) run[j] = acc[i][j][v];
                 if (interior) {
-                    store8<CDT>(p.c, off, lo, hi, 8, true);
+                    store_run<CDT, S::NT>(p.c, off, run, S::NT, true);
                 } else if (m < p.M && n < p.N) {
-                    const int nvalid = p.N - n < 8 ? p.N - n : 8;
+                    const int nvalid = p.N - n < S::NT ? p.N - n : S::NT;
                     if (CDT == MX_FP32 && p.accumulate) {
                         float *dst = (float *)p.c + off;
-                        for (int e = 0; e < 8 && e < nvalid; e++) atomicAdd(dst + e, e < 4 ? lo[e] : hi[e - 4]);
+                        for (int e = 0; e < S::NT && e < nvalid; e++) atomicAdd(dst + e, run[e]);
                     } else {
-                        store8<CDT>(p.c, off, lo, hi, nvalid, p.c_vec != 0);
+                        store_run<CDT, S::NT>(p.c, off, run, nvalid, p.c_vec != 0);
                     }
                 }
             }
@@ -199,6 +200,15 @@ struct DenseProblem {
 
 template <typename S, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
+    persistent_gemm<S, K512>(prob, smem);
+}
+
+// The same kernel body on a 128 x 128 tile with two workgroups resident per CU (4 waves each, one per SIMD and
+// workgroup): the second workgroup's K loop runs under the first one's epilogue, barrier waits and start-up.
+template <typename S, int CDT, int K512>
+__global__ __launch_bounds__(S::NTHR) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_pair_kernel(DenseArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
     persistent_gemm<S, K512>(prob, smem);
@@ -428,12 +438,32 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st) {
                                           : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
     if (rc != MX_OK) return rc;
     if (a.sk_tiles)
-        split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * S::MT)), block, 0, st>>>(a);
+        split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * S::MT)), dim3(S::NTHR), 0, st>>>(a);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
 // 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
 typedef GemmShape<256, 256, 4, 2> DenseShape;
+// 128 x 128 x 128 tile, 4 waves as 2 x 2: a wave owns 64 x 64, a lane 4 consecutive N; 73 KiB of LDS, two per CU.
+typedef GemmShape<128, 128, 2, 2> PairShape;
+
+template <int CDT>
+static int launch_pair(DenseArgs a, hipStream_t st) {
+    typedef PairShape S;
+    a.tiles_m = (a.M + S::BM - 1) / S::BM;
+    a.tiles_n = (a.N + S::BN - 1) / S::BN;
+    a.c_vec = aligned(a.c, 16) && (a.ldc * (CDT == MX_FP32 ? 4 : 2)) % 16 == 0;
+    const int mode = scale_mode(a);
+    const int64_t work = (int64_t)a.tiles_m * a.tiles_n * a.split_k;
+    a.dp_tiles = (int)work, a.sk_tiles = 0, a.sk_q = 0, a.sk_ws = nullptr;
+    const int wgs = 2 * num_cus();
+    dim3 grid((unsigned)(work < wgs ? work : wgs)), block(S::NTHR);
+    const int rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_pair_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+                   : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_pair_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
+                                          : launch_with_lds<gemm_nt_pair_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
+    if (rc != MX_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
 
 static bool tiled_ok(const DenseArgs &a) {
     const int64_t M = a.M, N = a.N;
@@ -443,8 +473,9 @@ static bool tiled_ok(const DenseArgs &a) {
 }
 
 template <int CDT>
-static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st) {
+static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool pair = false) {
     const int64_t M = a.M, N = a.N;
+    if (pair && tiled_ok(a) && a.split_k == 1 && !a.slice_ws) return launch_pair<CDT>(a, st);
     if (!tiled_ok(a)) {
         if (a.accumulate || a.a_ks || a.b_ks) return MX_EUNSUPPORTED;  // the element-wise kernel reads row-major only
         int64_t blocks = (M * N + 255) / 256;
@@ -680,7 +711,8 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     int rc = fill_args(a, aq, as, bq, bs, c, M, N, K, lda, ldas, ldb, ldbs, ldc);
     if (rc != MX_OK) return rc;
     const int split_k = epilogue >> 8;  // MX_EPI_SPLIT_K(n)
-    const int epi = epilogue & 0xFF;
+    const bool pair = (epilogue & MX_EPI_TILE_128) != 0;
+    const int epi = epilogue & 0x0F;
     if (epi != MX_EPI_NONE && epi != MX_EPI_ACCUMULATE) return MX_EUNSUPPORTED;
     if (epi == MX_EPI_ACCUMULATE && c_dtype != MX_FP32) return MX_EINVAL;
     if (split_k > 1 && epi != MX_EPI_ACCUMULATE) return MX_EINVAL;
@@ -695,8 +727,8 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     a.accumulate = epi == MX_EPI_ACCUMULATE;
     a.split_k = split_k > 1 ? split_k : 1;
     switch (c_dtype) {
-    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st);
-    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st);
-    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st);
+    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st, pair);
+    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st, pair);
+    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st, pair);
     }
 }

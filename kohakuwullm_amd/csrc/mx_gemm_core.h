@@ -83,7 +83,7 @@ struct GemmShape {
     static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
     static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B);
     static constexpr bool TWO_ROWS = BM + BN > NTHR;
-    static_assert(NT == 8, "8 sub-tiles along N give a lane 8 consecutive N: one 16-byte store");
+    static_assert(NT == 8 || NT == 4, "a lane's NT sub-tiles are NT consecutive N: one 16-byte (or 8-byte) store");
     static_assert(WTM % 16 == 0, "a wave's M extent must be a multiple of 16");
     static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "DMA rows must divide over the waves");
     static_assert(BM + BN <= 2 * NTHR, "scale loader assumes at most two rows per thread");
@@ -500,6 +500,33 @@ __device__ __forceinline__ void store8(void *c, int64_t off, const v4f &lo, cons
         } else {
             for (int i = 0; i < 8 && i < nvalid; i++) p[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
         }
+    }
+}
+
+// The same for a lane that owns NT consecutive N (NT = 8: store8; NT = 4: one 8-byte store of 16-bit values).
+template <int CDT, int NT>
+__device__ __forceinline__ void store_run(void *c, int64_t off, const float (&v)[NT], int nvalid, bool vec) {
+    if (NT == 8) {
+        store8<CDT>(c, off, v4f{v[0], v[1], v[2], v[3]}, v4f{v[NT - 4], v[NT - 3], v[NT - 2], v[NT - 1]}, nvalid, vec);
+    } else if (CDT == MX_FP32) {
+        float *p = (float *)c + off;
+        if (vec && nvalid >= 4) *(v4f *)p = v4f{v[0], v[1], v[2], v[3]};
+        else for (int i = 0; i < 4 && i < nvalid; i++) p[i] = v[i];
+    } else {
+        uint32_t w[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (CDT == MX_BF16) {
+                w[i] = pack2_bf16(v[2 * i], v[2 * i + 1]);
+            } else {
+                typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                h2 h = {(_Float16)v[2 * i], (_Float16)v[2 * i + 1]};
+                w[i] = __builtin_bit_cast(uint32_t, h);
+            }
+        }
+        uint16_t *p = (uint16_t *)c + off;
+        if (vec && nvalid >= 4) *(v2i *)p = v2i{(int)w[0], (int)w[1]};
+        else for (int i = 0; i < 4 && i < nvalid; i++) p[i] = (uint16_t)(w[i >> 1] >> ((i & 1) * 16));
     }
 }
 
