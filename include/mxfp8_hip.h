@@ -54,6 +54,10 @@ enum mx_epilogue {
 /* OR into `epilogue` of mx_gemm_nt: run on 128 x 128 tiles with two workgroups per compute unit instead of one
  * 256 x 256 tile (same product; a tiling choice kept selectable so the two can be timed against each other). */
 #define MX_EPI_TILE_128 0x10
+/* OR into `epilogue` of mx_gemm_nt: the 256 x 256 tile with its eight waves as two groups of four half a K stage
+ * apart (two barriers per stage) instead of all eight in lockstep.  Same product bit for bit; selectable so the
+ * two schedules can be timed against each other. */
+#define MX_EPI_PHASED 0x20
 /* OR into `epilogue` to cut K into n slices that run as independent tiles (needs
  * MX_EPI_ACCUMULATE and a caller-zeroed C): fills the GPU when M*N alone gives too few tiles. */
 #define MX_EPI_SPLIT_K(n) ((n) << 8)

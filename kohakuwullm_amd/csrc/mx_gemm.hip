@@ -34,6 +34,7 @@ struct DenseArgs {
     // row, panel kt at kt * a_ks, row m of it at m * 128 (lda is 128 then); b_ks likewise.  A K stage
     // of a tile is then one contiguous run instead of 256 rows a pitch apart.
     int64_t a_ks, b_ks;
+    int phased;  // which schedule wrote the fp32 partial tiles: it decides which part of a tile a wave owns
 };
 
 // Whether tile_of staggers the column walk (see there): up to 64 K stages per tile.
@@ -98,6 +99,13 @@ struct DenseProblem {
         return true;
     }
 
+    __device__ __forceinline__ const uint8_t *scale_row(const Tile &t, int r) const {
+        const int mrem = p.M - t.m0, nrem = p.N - t.n0;
+        if (r < S::BM) return p.as + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.ldas;
+        r = b_row_of_lds<S>(r - S::BM);
+        return p.bs + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldbs;
+    }
+
     __device__ __forceinline__ void context(const Tile &t, const Lane &L0, IssueCtx<S> &c) const {
         const Lane L = opaque(L0);
         c.a_base = p.aq + (int64_t)t.m0 * p.lda;
@@ -124,13 +132,28 @@ struct DenseProblem {
             int grow = brow < nrem ? brow : nrem - 1;
             c.b_voff[q] = (uint32_t)(grow * p.ldb) + chunk * 16;
         }
-        auto srow = [&](int r) -> const uint8_t * {
-            if (r < S::BM) return p.as + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.ldas;
-            r = b_row_of_lds<S>(r - S::BM);
-            return p.bs + (int64_t)(t.n0 + (r < nrem ? r : nrem - 1)) * p.ldbs;
-        };
-        c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
-        c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
+        c.srow0 = scale_row(t, L.tid < S::BM + S::BN ? L.tid : 0);
+        c.srow1 = S::TWO_ROWS ? scale_row(t, L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
+    }
+
+    // the phased schedule's description of a tile: bases, pitches and limits; the lanes rebuild their offsets from them
+    __device__ __forceinline__ void context(const Tile &t, const Lane &L0, PhasedCtx<S> &c) const {
+        const Lane L = opaque(L0);
+        c.a_base = p.aq + (int64_t)t.m0 * p.lda;
+        c.b_base = p.bq + (int64_t)t.n0 * p.ldb;
+        c.a_ks = p.a_ks ? p.a_ks : 128;
+        c.b_ks = p.b_ks ? p.b_ks : 128;
+        c.kt0 = t.kt0;
+        c.kt1 = t.kt1;
+        c.tail_bytes = p.K & 127;
+        c.tail_kt = c.tail_bytes ? p.K >> 7 : -1;
+        c.a_last = (p.M - t.m0 < S::BM ? p.M - t.m0 : S::BM) - 1;
+        c.b_last = (p.N - t.n0 < S::BN ? p.N - t.n0 : S::BN) - 1;
+        c.lda = (int)p.lda;
+        c.ldb = (int)p.ldb;
+        c.lanes(L);
+        c.srow0 = scale_row(t, L.tid);
+        c.srow1 = nullptr;
     }
 
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
@@ -205,6 +228,14 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
     persistent_gemm<S, K512>(prob, smem);
 }
 
+// The same tiles under the phased schedule (two groups of four waves half a K stage apart): MX_EPI_PHASED.
+template <typename S, int CDT, int K512>
+__global__ __launch_bounds__(S::NTHR) void gemm_nt_phased_kernel(DenseArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
+    persistent_gemm_phased<S, K512>(prob, smem);
+}
+
 // The same kernel body on a 128 x 128 tile with two workgroups resident per CU (4 waves each, one per SIMD and
 // workgroup): the second workgroup's K loop runs under the first one's epilogue, barrier waits and start-up.
 template <typename S, int CDT, int K512>
@@ -264,7 +295,7 @@ __global__ __launch_bounds__(S::NTHR) void split_reduce_kernel(DenseArgs p) {
     int tm, tn;
     tile_of(p.dp_tiles + local, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K), p.xcds);
     const int wave = tid >> 6, lane = tid & 63;
-    const int wm = wave / S::WGN, wn = wave % S::WGN;
+    const int wm = p.phased ? wave & 3 : wave / S::WGN, wn = p.phased ? wave >> 2 : wave % S::WGN;
     const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
 #pragma unroll
     for (int v = 0; v < 4; v++) {
@@ -294,7 +325,7 @@ __global__ __launch_bounds__(S::NTHR) void slice_reduce_kernel(DenseArgs p) {
     int tm, tn;
     tile_of(index, p.tiles_m, p.tiles_n, tm, tn, stagger_columns(p.K), p.xcds);
     const int wave = tid >> 6, lane = tid & 63;
-    const int wm = wave / S::WGN, wn = wave % S::WGN;
+    const int wm = p.phased ? wave & 3 : wave / S::WGN, wn = p.phased ? wave >> 2 : wave % S::WGN;
     const int n = tn * S::BN + wn * S::WTN + 8 * (lane & 15);
 #pragma unroll
     for (int v = 0; v < 4; v++) {
@@ -401,7 +432,7 @@ static int scale_mode(const DenseArgs &a) {
 }
 
 template <typename S, int CDT>
-static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st) {
+static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool phased = false) {
     a.tiles_m = (a.M + S::BM - 1) / S::BM;
     a.tiles_n = (a.N + S::BN - 1) / S::BN;
     const int esz = CDT == MX_FP32 ? 4 : 2;
@@ -433,9 +464,16 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st) {
         }
     }
     dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
-    const int rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
-                   : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
-                                          : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
+    int rc;
+    a.phased = phased ? 1 : 0;
+    if (phased)
+        rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+             : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
+                                    : launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
+    else
+        rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+             : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
+                                    : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
     if (rc != MX_OK) return rc;
     if (a.sk_tiles)
         split_reduce_kernel<S, CDT><<<dim3((unsigned)(a.sk_tiles * S::MT)), dim3(S::NTHR), 0, st>>>(a);
@@ -473,7 +511,7 @@ static bool tiled_ok(const DenseArgs &a) {
 }
 
 template <int CDT>
-static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool pair = false) {
+static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool pair = false, bool phased = false) {
     const int64_t M = a.M, N = a.N;
     if (pair && tiled_ok(a) && a.split_k == 1 && !a.slice_ws) return launch_pair<CDT>(a, st);
     if (!tiled_ok(a)) {
@@ -484,7 +522,7 @@ static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, b
                                                                                   a.lda, a.ldas, a.ldb, a.ldbs, a.ldc);
         return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
     }
-    return launch_tiled<DenseShape, CDT>(a, ws, ws_slots, st);
+    return launch_tiled<DenseShape, CDT>(a, ws, ws_slots, st, phased);
 }
 
 // Several products behind one launch, the eight XCDs shared out among them whole.  Every problem
@@ -637,6 +675,7 @@ static int fill_args(DenseArgs &a, const uint8_t *aq, const uint8_t *as, const u
     a.xcds = 8;
     a.a_ks = a_panels ? M * 128 : 0;
     a.b_ks = b_panels ? N * 128 : 0;
+    a.phased = 0;
     return MX_OK;
 }
 
@@ -711,7 +750,7 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     int rc = fill_args(a, aq, as, bq, bs, c, M, N, K, lda, ldas, ldb, ldbs, ldc);
     if (rc != MX_OK) return rc;
     const int split_k = epilogue >> 8;  // MX_EPI_SPLIT_K(n)
-    const bool pair = (epilogue & MX_EPI_TILE_128) != 0;
+    const bool pair = (epilogue & MX_EPI_TILE_128) != 0, phased = (epilogue & MX_EPI_PHASED) != 0;
     const int epi = epilogue & 0x0F;
     if (epi != MX_EPI_NONE && epi != MX_EPI_ACCUMULATE) return MX_EUNSUPPORTED;
     if (epi == MX_EPI_ACCUMULATE && c_dtype != MX_FP32) return MX_EINVAL;
@@ -727,8 +766,8 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     a.accumulate = epi == MX_EPI_ACCUMULATE;
     a.split_k = split_k > 1 ? split_k : 1;
     switch (c_dtype) {
-    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st, pair);
-    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st, pair);
-    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st, pair);
+    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st, pair, phased);
+    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st, pair, phased);
+    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st, pair, phased);
     }
 }

@@ -371,27 +371,34 @@ def test_workspace_is_the_callers(oracle, m, n, k):
     assert torch.equal(_mx().mxfp8_matmul_pq(a, sa, b, sb), split)  # the wrapper brings a full workspace
 
 
-@pytest.mark.parametrize("m,n,k", [(16384, 1536, 4096), (2048 + 130, 3000, 1536), (4096 + 256, 8192, 2048), (300, 520, 160)])
-def test_tile_128_equals_tile_256(oracle, m, n, k):
-    """MX_EPI_TILE_128 (128 x 128 tiles, two workgroups per CU) against the default 256 x 256 tiling: every element
-    contracts the same K sequence whichever tile computes it, so the two agree bit for bit; both are held to the
-    oracle on sampled rows (the last rows, in a ragged tile, among them)."""
+@pytest.mark.parametrize("m,n,k", [(16384, 1536, 4096), (2048 + 130, 3000, 1536), (4096 + 256, 8192, 2048), (300, 520, 160), (512, 768, 2048), (1536, 4096, 16384)])
+def test_tilings_and_schedules_agree(oracle, m, n, k):
+    """The 256 x 256 tile in lockstep (default), the same tile with its waves in two groups half a stage apart
+    (MX_EPI_PHASED) and 128 x 128 tiles with two workgroups per CU (MX_EPI_TILE_128): every element contracts the
+    same K sequence whichever computes it, so all three agree bit for bit; held to the oracle on sampled rows (the
+    last rows, in a ragged tile, among them).  With a workspace the default and the phased schedule may also split K
+    the same way: equal again."""
     from kohakuwullm_amd import _lib
 
     aq, as_, bq, bs = _operands(oracle, m, n, k)
     f8 = torch.float8_e4m3fn
     a, sa, b, sb = aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)
+    ws = _lib.gemm_workspace(a)
 
-    def run(epilogue, dtype=torch.bfloat16):
+    def run(epilogue, dtype=torch.bfloat16, workspace=None):
         c = torch.full((m, n), float("nan"), device=DEV, dtype=dtype)
         _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(),
-                    _lib.MX_DTYPE[dtype], m, n, k, k, k // 32, k, k // 32, n, epilogue, None, 0)
+                    _lib.MX_DTYPE[dtype], m, n, k, k, k // 32, k, k // 32, n, epilogue,
+                    None if workspace is None else workspace.data_ptr(), 0 if workspace is None else workspace.numel())
         return c
 
-    default, small = run(0), run(0x10)  # MX_EPI_TILE_128
+    default, phased, small = run(0), run(0x20), run(0x10)  # MX_EPI_PHASED, MX_EPI_TILE_128
     assert torch.isfinite(default.float()).all()
-    assert torch.equal(default, small)
-    assert torch.equal(run(0, torch.float32), run(0x10, torch.float32))
+    assert torch.equal(default, small) and torch.equal(default, phased)
+    assert torch.equal(run(0, torch.float32), run(0x10, torch.float32)) and torch.equal(run(0, torch.float32), run(0x20, torch.float32))
+    assert torch.equal(run(0, workspace=ws), run(0x20, workspace=ws))
     g = torch.Generator().manual_seed(SEED)
     rows = torch.cat([torch.randperm(m, generator=g)[:64], torch.arange(m - 40, m)])
-    assert oracle.rel_error(small[rows.to(DEV)].cpu(), oracle.gemm_nt(aq[rows], as_[rows], bq, bs)) < TOL_BF16
+    ref = oracle.gemm_nt(aq[rows], as_[rows], bq, bs)
+    for got in (small, phased, run(0x20, workspace=ws)):
+        assert oracle.rel_error(got[rows.to(DEV)].cpu(), ref) < TOL_BF16
