@@ -552,10 +552,72 @@ def run_quant(dev, iters: int) -> dict:
             "avg_us": total_ms / (len(rows_out) * iters) * 1e3}
 
 
+GEMM_SHAPES = ((16384, 8192, 1536), (16384, 1536, 4096), (16384, 4096, 1536), (16384, 1536, 8192), (8192, 1536, 16384),
+               (1536, 4096, 16384), (8192, 8192, 8192))  # the six products of BASELINE configs[1], and configs[4]'s
+GEMM_VARIANTS = (("tile256_lockstep", 0), ("tile256_phased", 0x20), ("tile128_pair", 0x10))  # MX_EPI_PHASED, MX_EPI_TILE_128
+
+
+def run_gemm_variants(dev, iters: int) -> dict:
+    """mx_gemm_nt alone on the benchmark's products, cold operands (rotating copies), in the shipped tiling/schedule and in
+    the two selectable alternatives: same product bit for bit, timed against each other."""
+    import torch
+
+    from kohakuwullm_amd import _lib
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator().manual_seed(SEED)
+    rows = []
+    for m, n, k in GEMM_SHAPES:
+        copies = max(2, min(8, (600 << 20) // ((m + n) * k)))
+        ops = []
+        for _ in range(copies):
+            a = torch.randn(m, k, generator=g).bfloat16().to(dev)
+            b = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(dev)
+            ops.append((*quantize_mx(a), *quantize_mx(b)))
+            del a, b
+        ws = _lib.gemm_workspace(ops[0][0])
+        c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+        row = {"shape": [m, n, k]}
+        first = None
+        for name, flag in GEMM_VARIANTS:
+            state = {"i": 0}
+
+            def call():
+                aq, sa, bq, sb = ops[state["i"] % copies]
+                state["i"] += 1
+                _lib.invoke("mx_gemm_nt", 0, aq, aq.data_ptr(), sa.data_ptr(), bq.data_ptr(), sb.data_ptr(), c.data_ptr(), 0,
+                            m, n, k, k, k // 32, k, k // 32, n, flag, ws.data_ptr(), ws.numel())
+
+            ts = _event_times(call, iters, warm=copies)
+            state["i"] = 0
+            call()
+            torch.cuda.synchronize()
+            if first is None:
+                first = c.clone()
+            row[name] = {"us_median": round(ts[len(ts) // 2] * 1e3, 1), "tflops_median": round(2.0 * m * n * k / ts[len(ts) // 2] / 1e9, 1),
+                         "tflops_best": round(2.0 * m * n * k / ts[0] / 1e9, 1), "equal_to_shipped": bool(torch.equal(c, first))}
+        rows.append(row)
+        del ops
+    return {"shapes": rows}
+
+
 def standalone_line(args, dev) -> dict:
     """--workload stream | peak | quant: one JSON line each, the same schema as the step workloads."""
     common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
               "vs_baseline": None, "data": "synthetic"}
+    if args.workload == "gemm":
+        res = run_gemm_variants(dev, max(args.steps, 20))
+        flops = sum(2.0 * m * n * k for m, n, k in GEMM_SHAPES)
+        secs = sum(r["tile256_lockstep"]["us_median"] for r in res["shapes"]) * 1e-6
+        peaks = measured_peaks(dev)
+        val = flops / secs / 1e12
+        return {"metric": "MXFP8 GEMM TFLOP/s (mx_gemm_nt alone, cold operands, shipped tiling)", "value": round(val, 1), "unit": "TFLOP/s",
+                "ms_per_step": round(secs * 1e3, 4), "dtype": "e4m3 x e4m3, ue8m0 scales, fp32 accumulate, bf16 out", **common,
+                "config": {"workload": "the six products of BASELINE configs[1] and the 8192^3 of configs[4], each alone; the shipped 256x256 "
+                                       "lockstep kernel against MX_EPI_PHASED and MX_EPI_TILE_128", **res},
+                "roofline": {"kernel": "gemm_nt_kernel", "bound": "mfma", "achieved": round(val, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(val / MFMA_PEAK_TFLOPS, 4), "traffic": None, "peak_measured": peaks["mfma_tflops"],
+                             "frac_of_measured": round(val / peaks["mfma_tflops"], 4)}}
     if args.workload == "stream":
         bw = measure_stream(dev, iters=max(args.steps, 10))
         best = max(v["best"] for v in bw.values())
@@ -592,9 +654,10 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="ffn",
-                    choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh", "heads", "quant", "stream", "peak"),
+                    choices=("ffn", "attn", "moe", "outlier", "norm", "dispatch", "refresh", "heads", "quant", "gemm", "stream", "peak"),
                     help="ffn (default) is the configuration the headline metric is quoted on; quant: the stand-alone "
-                         "quantizers; stream / peak: the device's measured bandwidth and MFMA rate")
+                         "quantizers; gemm: mx_gemm_nt alone in its three tilings/schedules; stream / peak: the device's "
+                         "measured bandwidth and MFMA rate")
     ap.add_argument("--routing", default="draws", choices=("draws", "ranked"),
                     help="moe: per-expert loads drawn i.i.d. Zipf (six full experts with the fixed seed) or Zipf by rank (59 live experts)")
     ap.add_argument("--samples", type=int, default=0,
@@ -615,7 +678,7 @@ def main() -> None:
 
     dev = torch.device("cuda:0")
     _lib.check(_lib.load().mx_device_supported(0), "mx_device_supported")
-    if args.workload in ("quant", "stream", "peak"):
+    if args.workload in ("quant", "gemm", "stream", "peak"):
         print(json.dumps(standalone_line(args, dev)))
         return
     step, gflop, desc, refresh = build_workload(args.workload, dev, args.routing)
