@@ -547,6 +547,20 @@ STREAM_METRICS = {
 QUANT_SHAPES = ((16384, 1536), (16384, 4096), (32768, 2048), (8192, 8192))  # activations of BASELINE configs[1], [1], [2], [4]
 
 
+def _dequant(q, s):
+    """fp32 values of an MXFP8 pair (codes (R, K), scale bytes (R, K/32)) with torch ops on the tensors' device."""
+    import torch
+
+    scale = torch.exp2(s.to(torch.float32) - 127.0).repeat_interleave(32, dim=1)
+    return q.to(torch.float32) * scale
+
+
+def _rel_error(got, want) -> float:
+    """Relative Frobenius distance, accumulated in fp64 (the reference's accuracy figure, bench/core/timing.py:201-206)."""
+    d = (got.double() - want.double()).norm()
+    return float(d / want.double().norm())
+
+
 def run_quant(dev, iters: int) -> dict:
     """The stand-alone quantizers (rows, columns, both) on the activation shapes, cold: every launch reads a copy of
     the input that left the 256 MB last-level cache several launches ago.  Per kernel and shape: algorithmic bytes
@@ -572,9 +586,13 @@ def run_quant(dev, iters: int) -> dict:
             ts = _event_times(call, iters, warm=copies)
             nbytes = m * k * per_elem
             med, best = ts[len(ts) // 2], ts[0]
+            # accuracy in the same row: what the cast loses, dequantized on the device against the 16-bit input
+            out = fn(xs[0])
+            loss = _rel_error(_dequant(out[0], out[1]) if name != "cols" else _dequant(out[0], out[1]).t(), xs[0])
+            del out
             rows_out.append({"kernel": f"quantize_mx_{name}", "shape": [m, k], "us_median": round(med * 1e3, 2),
                              "us_best": round(best * 1e3, 2), "gbs_median": round(nbytes / med / 1e6, 1),
-                             "gbs_best": round(nbytes / best / 1e6, 1)})
+                             "gbs_best": round(nbytes / best / 1e6, 1), "rel_error_of_cast": round(loss, 5)})
             total_bytes += nbytes * len(ts)
             total_ms += sum(ts)
         del xs
@@ -624,6 +642,9 @@ def run_gemm_variants(dev, iters: int) -> dict:
             torch.cuda.synchronize()
             if first is None:
                 first = c.clone()
+                # accuracy in the same row: against torch's fp32 matmul of the dequantized operands, on the device
+                aq, sa, bq, sb = ops[0]
+                row["rel_error"] = round(_rel_error(first, _dequant(aq, sa) @ _dequant(bq, sb).t()), 6)
             row[name] = {"us_median": round(ts[len(ts) // 2] * 1e3, 1), "tflops_median": round(2.0 * m * n * k / ts[len(ts) // 2] / 1e9, 1),
                          "tflops_best": round(2.0 * m * n * k / ts[0] / 1e9, 1), "equal_to_shipped": bool(torch.equal(c, first))}
         rows.append(row)
