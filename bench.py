@@ -278,7 +278,10 @@ def measure_mfma(dev, iters: int = 4000, repeats: int = 5) -> dict:
     sink = torch.empty(cus * 512, dtype=torch.float32, device=dev)
     st = torch.cuda.current_stream(dev).cuda_stream
     out = {}
-    for wide, shape, flop in ((0, "16x16x128", 2.0 * 16 * 16 * 128), (1, "32x32x64", 2.0 * 32 * 32 * 64)):
+    for wide, shape, flop in ((0, "16x16x128", 2.0 * 16 * 16 * 128), (1, "32x32x64", 2.0 * 32 * 32 * 64),
+                              (2, "16x16x128_one_wave_per_simd", 2.0 * 16 * 16 * 128),
+                              (4, "16x16x128_scales_in_registers", 2.0 * 16 * 16 * 128),
+                              (6, "16x16x128_scales_in_registers_one_wave_per_simd", 2.0 * 16 * 16 * 128)):
         for random, label in ((1, "hashed"), (0, "zeros")):
             count = []
 
@@ -602,12 +605,13 @@ def run_quant(dev, iters: int) -> dict:
 
 GEMM_SHAPES = ((16384, 8192, 1536), (16384, 1536, 4096), (16384, 4096, 1536), (16384, 1536, 8192), (8192, 1536, 16384),
                (1536, 4096, 16384), (8192, 8192, 8192))  # the six products of BASELINE configs[1], and configs[4]'s
-GEMM_VARIANTS = (("tile256_lockstep", 0), ("tile256_phased", 0x20), ("tile128_pair", 0x10))  # MX_EPI_PHASED, MX_EPI_TILE_128
+GEMM_VARIANTS = (("tile256_lockstep", 0), ("tile256_phased", 0x20), ("tile128_pair", 0x10),
+                 ("tile256_wide_waves", 0x40))  # MX_EPI_PHASED, MX_EPI_TILE_128, MX_EPI_WIDE_WAVES
 
 
 def run_gemm_variants(dev, iters: int) -> dict:
     """mx_gemm_nt alone on the benchmark's products, cold operands (rotating copies), in the shipped tiling/schedule and in
-    the two selectable alternatives: same product bit for bit, timed against each other."""
+    the selectable alternatives: same product bit for bit, timed against each other."""
     import torch
 
     from kohakuwullm_amd import _lib

@@ -58,6 +58,10 @@ enum mx_epilogue {
  * apart (two barriers per stage) instead of all eight in lockstep.  Same product bit for bit; selectable so the
  * two schedules can be timed against each other. */
 #define MX_EPI_PHASED 0x20
+/* OR into `epilogue` of mx_gemm_nt: the 256 x 256 tile on four waves, one per SIMD, 128 x 128 each, accumulators in
+ * the accumulation registers and the next stage's first operands read under the current stage's last MFMAs.  Same
+ * product bit for bit; selectable so the schedules can be timed against each other. */
+#define MX_EPI_WIDE_WAVES 0x40
 /* OR into `epilogue` to cut K into n slices that run as independent tiles (needs
  * MX_EPI_ACCUMULATE and a caller-zeroed C): fills the GPU when M*N alone gives too few tiles. */
 #define MX_EPI_SPLIT_K(n) ((n) << 8)
@@ -483,9 +487,9 @@ int mx_combine_routed_backward(const void *grad_out, int64_t ldg, const void *ro
 int mx_ubench_stream(int kind, const void *a, const void *b, void *c, int64_t out_bytes, void *stream);
 
 /*
- * Register-resident loop of the block-scaled fp8 MFMA (wide == 0: v_mfma_scale_f32_16x16x128_f8f6f4 with
- * 8 independent accumulator tiles per wave, wide != 0: ..._32x32x64_... with 4), 8 waves on every CU,
- * `iters` rounds; operands zero or (random != 0) a per-lane hash.  Returns the number of MFMA
+ * Register-resident loop of the block-scaled fp8 MFMA (bit 0 of wide clear: v_mfma_scale_f32_16x16x128_f8f6f4
+ * with 8 independent accumulator tiles per wave, set: ..._32x32x64_... with 4), 8 waves on every CU (bit 1 of
+ * wide set: 4 waves, one per SIMD), `iters` rounds; operands zero or (random != 0) a per-lane hash.  Returns the number of MFMA
  * instructions the launch issues (each 2 * 16*16*128 = 65536 or 2 * 32*32*64 = 131072 FLOP) or a
  * negative mx_status.  out: one float per launched thread (512 x CUs).  The reference's rule for a
  * compute ceiling: measured from registers with independent accumulators

@@ -236,6 +236,15 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_phased_kernel(DenseArgs args)
     persistent_gemm_phased<S, K512>(prob, smem);
 }
 
+// The same tiles under the wide-wave schedule (four waves, one per SIMD, 128 x 128 each, accumulators in the
+// accumulation registers, the next stage's first fragments read under the last MFMAs of the current one).
+template <typename S, int CDT, int K512>
+__global__ __launch_bounds__(S::NTHR) void gemm_nt_wide_kernel(DenseArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
+    persistent_gemm_wide<S, K512>(prob, smem);
+}
+
 // The same kernel body on a 128 x 128 tile with two workgroups resident per CU (4 waves each, one per SIMD and
 // workgroup): the second workgroup's K loop runs under the first one's epilogue, barrier waits and start-up.
 template <typename S, int CDT, int K512>
@@ -466,7 +475,11 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
     dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
     int rc;
     a.phased = phased ? 1 : 0;
-    if (phased)
+    if constexpr (S::NW == 4)
+        rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_wide_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+             : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_wide_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
+                                    : launch_with_lds<gemm_nt_wide_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
+    else if (phased)
         rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
              : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
                                     : launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
@@ -484,6 +497,8 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
 typedef GemmShape<256, 256, 4, 2> DenseShape;
 // 128 x 128 x 128 tile, 4 waves as 2 x 2: a wave owns 64 x 64, a lane 4 consecutive N; 73 KiB of LDS, two per CU.
 typedef GemmShape<128, 128, 2, 2> PairShape;
+// 256 x 256 x 128 tile, 4 waves as 2 x 2, one per SIMD: a wave owns 128 x 128 (the wide-wave schedule).
+typedef GemmShape<256, 256, 2, 2> WideShape;
 
 template <int CDT>
 static int launch_pair(DenseArgs a, hipStream_t st) {
@@ -511,9 +526,11 @@ static bool tiled_ok(const DenseArgs &a) {
 }
 
 template <int CDT>
-static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool pair = false, bool phased = false) {
+static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool pair = false, bool phased = false,
+                         bool wide = false) {
     const int64_t M = a.M, N = a.N;
     if (pair && tiled_ok(a) && a.split_k == 1 && !a.slice_ws) return launch_pair<CDT>(a, st);
+    if (wide && tiled_ok(a)) return launch_tiled<WideShape, CDT>(a, ws, ws_slots, st, false);
     if (!tiled_ok(a)) {
         if (a.accumulate || a.a_ks || a.b_ks) return MX_EUNSUPPORTED;  // the element-wise kernel reads row-major only
         int64_t blocks = (M * N + 255) / 256;
@@ -751,6 +768,7 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     if (rc != MX_OK) return rc;
     const int split_k = epilogue >> 8;  // MX_EPI_SPLIT_K(n)
     const bool pair = (epilogue & MX_EPI_TILE_128) != 0, phased = (epilogue & MX_EPI_PHASED) != 0;
+    const bool wide = (epilogue & MX_EPI_WIDE_WAVES) != 0;
     const int epi = epilogue & 0x0F;
     if (epi != MX_EPI_NONE && epi != MX_EPI_ACCUMULATE) return MX_EUNSUPPORTED;
     if (epi == MX_EPI_ACCUMULATE && c_dtype != MX_FP32) return MX_EINVAL;
@@ -766,8 +784,8 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     a.accumulate = epi == MX_EPI_ACCUMULATE;
     a.split_k = split_k > 1 ? split_k : 1;
     switch (c_dtype) {
-    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st, pair, phased);
-    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st, pair, phased);
-    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st, pair, phased);
+    case MX_BF16: return gemm_dispatch<MX_BF16>(a, ws, ws_slots, st, pair, phased, wide);
+    case MX_FP16: return gemm_dispatch<MX_FP16>(a, ws, ws_slots, st, pair, phased, wide);
+    default: return gemm_dispatch<MX_FP32>(a, ws, ws_slots, st, pair, phased, wide);
     }
 }

@@ -478,6 +478,212 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// The wide-wave schedule (dense kernels, GemmShape<256, 256, 2, 2>): four waves per workgroup, one per SIMD, each
+// owning 128 x 128 of the tile.  A wave then has the whole register file of its SIMD: the 64 accumulator tiles live
+// in the 256 accumulation registers and the vector registers hold TWO sets of A fragments, so the first fragments of
+// stage k + 1 are read while the last MFMAs of stage k run, and no wave ever stands at a barrier with an empty pipe
+// and its operands still in LDS (the lockstep schedule's read burst after the barrier and its one-wave tail).
+//
+// One barrier per stage, in front of step 6 of 8:
+//   * steps 0-3: the wave issues its 16 copies of stage k + 1 into the other buffer (free: every wave passed the
+//     barrier of stage k - 1 after its last read of that buffer);
+//   * step j reads B fragment j + 1, step 5 reads fragments 6 AND 7: nothing of this stage's buffer is left to read;
+//   * in front of step 6: wait for those reads and for the wave's own copies, barrier.  Behind it stage k + 1's data
+//     is visible to all and this stage's buffer is dead for all, so the copies of stage k + 2 may overwrite it from
+//     the next stage's step 0 on;
+//   * steps 6-7 (512 clocks of MFMA) cover the reads of stage k + 1's eight A fragments (into the other set) and its
+//     first B fragment.
+// The last stage of a tile has no such barrier: the next tile's first stage, already in flight, is published by the
+// barrier behind the epilogue as in the lockstep schedule, and the tile reads its first fragments itself.
+// B fragments rotate through four buffers (fragment j in buffer j % 4), so buffer 0 is free for the next stage's
+// first fragment from step 5 on.
+//
+// Measured (MX_EPI_WIDE_WAVES; results bit-identical to the lockstep schedule): slower, 2.1 against 2.7 PFLOP/s at
+// 8192^3.  A wave alone on its SIMD does not issue this MFMA every 32 clocks in a GEMM's operand pattern (eight A
+// fragments against one B fragment, accumulators in the accumulation registers): with the copies and all LDS reads
+// taken out of the stage it still needs 51 clocks per MFMA, and every copy it hands to the texture path is time in
+// which its SIMD issues nothing.  Two waves per SIMD fill each other's gaps; the lockstep schedule stays the default.
+template <typename S, int OPSEL>
+__device__ __forceinline__ void wide_stage(const uint8_t *__restrict__ la_n, const uint8_t *__restrict__ lb,
+                                           const uint8_t *__restrict__ lb_n, int a_lo, int a_hi, int b_lo, int b_hi,
+                                           const int (&sa)[S::MT], const int (&sb)[S::NT], v4f (&acc)[S::MT][S::NT],
+                                           const v8i (&afr)[S::MT], v8i (&afr_n)[S::MT], v8i (&bfr)[4], const IssueCtx<S> &c,
+                                           const Lane &L, int kt_next, uint8_t *ldsA, uint8_t *ldsB, int buf_next, bool more) {
+    static_assert(S::NT == 8, "the step numbers below are those of eight B fragments");
+    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt_next * c.a_ks);
+    const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt_next * c.b_ks);
+    const uint32_t wa = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf_next * S::DATA_A + L.wave * 1024);
+    const uint32_t wb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf_next * S::DATA_B + L.wave * 1024);
+    constexpr int NQ = S::QA + S::QB, COPY_STEPS = 4;
+    auto issue = [&](int q) {
+        if (q < S::QA) dma16(ga, c.a_voff[q] - tail_fix<S>(c, L, kt_next, q), wa + q * S::NW * 1024);
+        else dma16(gb, c.b_voff[q - S::QA] - tail_fix<S>(c, L, kt_next, q - S::QA), wb + (q - S::QA) * S::NW * 1024);
+    };
+    auto read_b = [&](const uint8_t *base, int frag, v8i &dst) {
+        v4i lo = *(const v4i *)(base + b_lo + frag * (16 * 128));
+        v4i hi = *(const v4i *)(base + b_hi + frag * (16 * 128));
+        dst = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < S::NT; j++) {
+        if (j < 5) read_b(lb, j + 1, bfr[(j + 1) & 3]);
+        if (j == 5) {
+            read_b(lb, 6, bfr[2]);
+            read_b(lb, 7, bfr[3]);
+        }
+        if (j < COPY_STEPS) {
+#pragma unroll
+            for (int q = j * NQ / COPY_STEPS; q < (j + 1) * NQ / COPY_STEPS; q++) issue(q);
+        }
+        // fragments 6 and 7 are waited for on both paths, so that behind the branch nothing older than the next stage's
+        // reads is outstanding and steps 6 and 7 do not wait for those
+        if (j == 6) wait_vm_allow_c<63>();
+        if (j == 6 && more) {
+            wait_vm_allow_c<0>();  // this wave's copies of the next stage have landed
+            __syncthreads();
+            read_b(lb_n, 0, bfr[0]);
+#pragma unroll
+            for (int i = 0; i < S::MT; i++) {
+                v4i lo = *(const v4i *)(la_n + a_lo + i * (16 * 128));
+                v4i hi = *(const v4i *)(la_n + a_hi + i * (16 * 128));
+                afr_n[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < S::MT; i++)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(afr[i], bfr[j & 3], acc[i][j], 0, 0, OPSEL, sa[i],
+                                                                         OPSEL, sb[j]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // pins the MFMAs in front of whatever follows the stage; "a": the accumulators stay in the accumulation registers
+#pragma unroll
+    for (int i = 0; i < S::MT; i++)
+#pragma unroll
+        for (int j = 0; j < S::NT; j++) asm volatile("" : "+a"(acc[i][j]));
+}
+
+template <typename S, int K512, typename P>
+__device__ __forceinline__ void persistent_gemm_wide(P &prob, uint8_t *smem) {
+    static_assert(S::NW == 4 && !P::EARLY_WAIT, "one wave per SIMD; dense epilogues");
+    uint8_t *const ldsA = smem;
+    uint8_t *const ldsB = smem + 2 * S::DATA_A;
+    uint32_t *const ldsSA = (uint32_t *)(smem + 2 * (S::DATA_A + S::DATA_B));
+    uint32_t *const ldsSB = ldsSA + 2 * 4 * S::PA;
+
+    const Lane L = lane_of<S>();
+    const bool has_row0 = L.tid < S::BM + S::BN;
+    const int kb_end = prob.kb_end;
+    const int a_row = L.wm * S::WTM + L.r16;
+    const int b_row = L.wn * S::WTN + L.r16;
+    const int a_rd = a_row * 128 + ((L.g ^ swz_a(a_row)) << 4);
+    const int b_rd = b_row * 128 + ((L.g ^ swz_a(b_row)) << 4);
+
+    typename P::Tile cur, nxt;
+    if (!prob.next(cur)) return;
+    bool has_next = prob.next(nxt);
+    IssueCtx<S> ctx;
+    prob.context(cur, L, ctx);
+
+    int gstage = 0, gsuper = 0;
+    {
+        uint32_t d0[4], d1[4];
+        if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);
+        if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);
+        issue_stage<S>(ctx, L, ctx.kt0, ldsA, ldsB, 0);
+        if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
+        if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
+    }
+    wait_vm_allow_c<0>();
+    __syncthreads();
+
+    v4f acc[S::MT][S::NT];
+    v8i afr[2][S::MT], bfr[4];
+    while (true) {
+#pragma unroll
+        for (int i = 0; i < S::MT; i++)
+#pragma unroll
+            for (int j = 0; j < S::NT; j++) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+        // the tile's first fragments (every later stage finds its own already in registers)
+        {
+            const uint8_t *la = ldsA + (gstage & 1) * S::DATA_A, *lb = ldsB + (gstage & 1) * S::DATA_B;
+            v4i lo = *(const v4i *)(lb + b_rd);
+            v4i hi = *(const v4i *)(lb + (b_rd ^ 64));
+            bfr[0] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int i = 0; i < S::MT; i++) {
+                v4i l2 = *(const v4i *)(la + a_rd + i * (16 * 128));
+                v4i h2 = *(const v4i *)(la + (a_rd ^ 64) + i * (16 * 128));
+                afr[0][i] = __builtin_shufflevector(l2, h2, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+
+        const int kt0 = ctx.kt0, KT = ctx.kt1 - ctx.kt0;
+        const int nsuper = (KT + 3) >> 2;
+        uint32_t d0[4], d1[4];
+        for (int ss = 0; ss < nsuper; ss++) {
+            const int sbuf = gsuper & 1;
+            int sa[S::MT], sb[S::NT];
+#pragma unroll
+            for (int i = 0; i < S::MT; i++) sa[i] = (int)ldsSA[(sbuf * 4 + L.g) * S::PA + a_row + 16 * i];
+#pragma unroll
+            for (int j = 0; j < S::NT; j++) sb[j] = (int)ldsSB[(sbuf * 4 + L.g) * S::PB + b_row + 16 * j];
+
+#define MX_WSTAGE(SIDX)                                                                                       \
+    {                                                                                                         \
+        const int k = ss * 4 + SIDX;                                                                          \
+        if (k < KT) {                                                                                         \
+            const int buf = gstage & 1;                                                                       \
+            const bool last = k + 1 == KT;                                                                    \
+            int kt_issue = kt0 + k + 1;                                                                       \
+            if (!last) {                                                                                      \
+                if (SIDX == 3) {                                                                              \
+                    if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, sbuf ^ 1, d0);                          \
+                    if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, sbuf ^ 1, d1);             \
+                }                                                                                             \
+                if (SIDX == 0 && ss + 1 < nsuper) {                                                           \
+                    if (has_row0) load_scales<K512>(ctx.srow0, (kt0 + (ss + 1) * 4) * 4, kb_end, d0);         \
+                    if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, (kt0 + (ss + 1) * 4) * 4, kb_end, d1);      \
+                }                                                                                             \
+            } else if (has_next) {                                                                            \
+                prob.context(nxt, L, ctx);                                                                    \
+                if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);                          \
+                if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);                       \
+                kt_issue = ctx.kt0;                                                                           \
+            } else {                                                                                          \
+                kt_issue = kt0 + k;                                                                           \
+            }                                                                                                 \
+            wide_stage<S, SIDX>(ldsA + (buf ^ 1) * S::DATA_A, ldsB + buf * S::DATA_B, ldsB + (buf ^ 1) * S::DATA_B, a_rd,      \
+                                a_rd ^ 64, b_rd, b_rd ^ 64, sa, sb, acc, afr[SIDX & 1], afr[(SIDX + 1) & 1], bfr, ctx, L,      \
+                                kt_issue, ldsA, ldsB, buf ^ 1, !last);                                        \
+            gstage++;                                                                                         \
+        }                                                                                                     \
+    }
+            MX_WSTAGE(0)
+            MX_WSTAGE(1)
+            MX_WSTAGE(2)
+            MX_WSTAGE(3)
+#undef MX_WSTAGE
+            gsuper++;
+        }
+        const int lastbuf = (gstage - 1) & 1;
+        const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B,
+                                            (uint8_t *)(ldsSA + ((gsuper - 1) & 1) * 4 * S::PA)});
+        if (has_next) {
+            if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
+            if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);
+        }
+        if (!has_next) break;
+        if (stores == P::NST && P::NST <= 63) wait_vm_allow_c<(P::NST <= 63 ? P::NST : 0)>();
+        else wait_vm_allow_c<0>();
+        __syncthreads();
+        cur = nxt;
+        has_next = prob.next(nxt);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // The phased schedule (dense kernels).  Same tile, same LDS layout, same K-stage arithmetic as
 // persistent_gemm above, but the eight waves run as two groups of four -- one wave of each group on
 // every SIMD -- HALF A STAGE APART: waves 0-3 (group 0, the tile's columns 0-127) begin a stage when

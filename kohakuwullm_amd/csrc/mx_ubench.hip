@@ -66,7 +66,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_kernel(const v4i *__res
 // Register-resident block-scaled fp8 MFMA loop: ACCS independent accumulator tiles per wave, operands that never
 // change, no memory traffic.  `random` fills the operand registers with a per-lane hash (switching activity of
 // real data) instead of zeros: the part's clock, and with it this peak, depends on what the multipliers see.
-template <bool WIDE>  // false: 16x16x128 (4 accumulator registers), true: 32x32x64 (16)
+template <bool WIDE, bool VSCALE = false>  // WIDE false: 16x16x128 (4 accumulator registers), true: 32x32x64 (16)
 __global__ __launch_bounds__(512) void mfma_peak_kernel(int iters, int random, float *out) {
     typedef float v16f __attribute__((ext_vector_type(16)));
     constexpr int ACCS = WIDE ? 4 : 8;
@@ -82,6 +82,14 @@ __global__ __launch_bounds__(512) void mfma_peak_kernel(int iters, int random, f
             a[k][i] = random ? (int)h : 0;
             b[k][i] = random ? (int)((h * 0x27D4EB2Fu) & 0xF7F7F7F7u) : 0;
         }
+    // VSCALE: the scale bytes come from vector registers the compiler cannot see through (as in a GEMM, where they
+    // are data), one register per accumulator tile, instead of an inline constant
+    int sc[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        sc[j] = 0x7F7F7F7F;
+        if (VSCALE) asm volatile("" : "+v"(sc[j]));
+    }
     float sum = 0.f;
     if (!WIDE) {
         v4f acc[ACCS];
@@ -90,8 +98,10 @@ __global__ __launch_bounds__(512) void mfma_peak_kernel(int iters, int random, f
         for (int it = 0; it < iters; it++) {
 #pragma unroll
             for (int j = 0; j < ACCS; j++)
-                acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[j & 1], b[(j >> 1) & 1], acc[j], 0, 0, 0, 0x7F7F7F7F, 0,
-                                                                          0x7F7F7F7F);
+                acc[j] = VSCALE ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[j & 1], b[(j >> 1) & 1], acc[j], 0, 0, 0, sc[j], 0,
+                                                                                   sc[(j + 3) & 7])
+                                : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[j & 1], b[(j >> 1) & 1], acc[j], 0, 0, 0,
+                                                                                   0x7F7F7F7F, 0, 0x7F7F7F7F);
         }
 #pragma unroll
         for (int j = 0; j < ACCS; j++) sum += acc[j][0] + acc[j][3];
@@ -142,9 +152,13 @@ extern "C" int64_t mx_ubench_mfma(int wide, int iters, int random, float *out, i
     if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     const int cus = num_cus();
     if (out_floats < (int64_t)cus * 512) return MX_EINVAL;
-    if (wide) mfma_peak_kernel<true><<<dim3((unsigned)cus), dim3(512), 0, st>>>(iters, random, out);
-    else mfma_peak_kernel<false><<<dim3((unsigned)cus), dim3(512), 0, st>>>(iters, random, out);
+    // bit 0 of `wide`: the 32x32x64 form; bit 1: four waves per CU (one per SIMD) instead of eight; bit 2 (16x16x128
+    // only): scale bytes from vector registers instead of an inline constant
+    const int waves = (wide & 2) ? 4 : 8;
+    if (wide & 1) mfma_peak_kernel<true><<<dim3((unsigned)cus), dim3(waves * 64), 0, st>>>(iters, random, out);
+    else if (wide & 4) mfma_peak_kernel<false, true><<<dim3((unsigned)cus), dim3(waves * 64), 0, st>>>(iters, random, out);
+    else mfma_peak_kernel<false><<<dim3((unsigned)cus), dim3(waves * 64), 0, st>>>(iters, random, out);
     if (hipGetLastError() != hipSuccess) return MX_ELAUNCH;
-    // MFMA instructions issued by the launch: workgroups x 8 waves x iterations x accumulators per wave
-    return (int64_t)cus * 8 * iters * (wide ? 4 : 8);
+    // MFMA instructions issued by the launch: workgroups x waves x iterations x accumulators per wave
+    return (int64_t)cus * waves * iters * ((wide & 1) ? 4 : 8);
 }

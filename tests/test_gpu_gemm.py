@@ -374,10 +374,10 @@ def test_workspace_is_the_callers(oracle, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(16384, 1536, 4096), (2048 + 130, 3000, 1536), (4096 + 256, 8192, 2048), (300, 520, 160), (512, 768, 2048), (1536, 4096, 16384)])
 def test_tilings_and_schedules_agree(oracle, m, n, k):
     """The 256 x 256 tile in lockstep (default), the same tile with its waves in two groups half a stage apart
-    (MX_EPI_PHASED) and 128 x 128 tiles with two workgroups per CU (MX_EPI_TILE_128): every element contracts the
-    same K sequence whichever computes it, so all three agree bit for bit; held to the oracle on sampled rows (the
-    last rows, in a ragged tile, among them).  With a workspace the default and the phased schedule may also split K
-    the same way: equal again."""
+    (MX_EPI_PHASED), 128 x 128 tiles with two workgroups per CU (MX_EPI_TILE_128) and the 256 x 256 tile on four
+    waves of 128 x 128 (MX_EPI_WIDE_WAVES): every element contracts the same K sequence whichever computes it, so
+    all four agree bit for bit; held to the oracle on sampled rows (the last rows, in a ragged tile, among them).
+    With a workspace the default, the phased and the wide-wave schedule may also split K the same way: equal again."""
     from kohakuwullm_amd import _lib
 
     aq, as_, bq, bs = _operands(oracle, m, n, k)
@@ -392,13 +392,14 @@ def test_tilings_and_schedules_agree(oracle, m, n, k):
                     None if workspace is None else workspace.data_ptr(), 0 if workspace is None else workspace.numel())
         return c
 
-    default, phased, small = run(0), run(0x20), run(0x10)  # MX_EPI_PHASED, MX_EPI_TILE_128
+    default, phased, small, wide = run(0), run(0x20), run(0x10), run(0x40)  # MX_EPI_PHASED, MX_EPI_TILE_128, MX_EPI_WIDE_WAVES
     assert torch.isfinite(default.float()).all()
-    assert torch.equal(default, small) and torch.equal(default, phased)
+    assert torch.equal(default, small) and torch.equal(default, phased) and torch.equal(default, wide)
     assert torch.equal(run(0, torch.float32), run(0x10, torch.float32)) and torch.equal(run(0, torch.float32), run(0x20, torch.float32))
-    assert torch.equal(run(0, workspace=ws), run(0x20, workspace=ws))
+    assert torch.equal(run(0, torch.float32), run(0x40, torch.float32)) and torch.equal(run(0, torch.float16), run(0x40, torch.float16))
+    assert torch.equal(run(0, workspace=ws), run(0x20, workspace=ws)) and torch.equal(run(0, workspace=ws), run(0x40, workspace=ws))
     g = torch.Generator().manual_seed(SEED)
     rows = torch.cat([torch.randperm(m, generator=g)[:64], torch.arange(m - 40, m)])
     ref = oracle.gemm_nt(aq[rows], as_[rows], bq, bs)
-    for got in (small, phased, run(0x20, workspace=ws)):
+    for got in (small, phased, wide, run(0x20, workspace=ws)):
         assert oracle.rel_error(got[rows.to(DEV)].cpu(), ref) < TOL_BF16
