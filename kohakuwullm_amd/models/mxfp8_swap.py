@@ -190,22 +190,22 @@ def _convert_declared(parent: nn.Module, prefix: str, census: _Census, convert_d
     if not open_cases:
         return
     if not census.wanted(prefix):
-        verdict = lambda entry: ("out_of_scope", None)  # noqa: E731
+        ruling = lambda entry: ("out_of_scope", None)  # noqa: E731
     elif any(entry.refusal for _, entry in open_cases):
         # one refused tensor keeps the whole module in 16 bits; its siblings point at it
         sibling = f"a sibling tensor in {prefix or '<root>'} is refused"
-        verdict = lambda entry: ("skipped", entry.refusal or sibling)  # noqa: E731
+        ruling = lambda entry: ("skipped", entry.refusal or sibling)  # noqa: E731
     elif not convert_declared:
-        verdict = lambda entry: ("unreached", "the caller passed convert_declared=False")  # noqa: E731
+        ruling = lambda entry: ("unreached", "the caller passed convert_declared=False")  # noqa: E731
     elif not callable(getattr(parent, CONVERT, None)):
         missing = f"{type(parent).__name__} declares it fp8-eligible but has no {CONVERT}()"
-        verdict = lambda entry: ("unreached", missing)  # noqa: E731
+        ruling = lambda entry: ("unreached", missing)  # noqa: E731
     else:
         getattr(parent, CONVERT)()
         census.report.modules.append(prefix)
-        verdict = lambda entry: ("fp8", None)  # noqa: E731
+        ruling = lambda entry: ("fp8", None)  # noqa: E731
     for where, entry in open_cases:
-        outcome, why = verdict(entry)
+        outcome, why = ruling(entry)
         census.book(outcome, where, entry.mac_per_token, why)
 
 
