@@ -611,7 +611,7 @@ GEMM_VARIANTS = (("tile256_lockstep", 0), ("tile256_phased", 0x20), ("tile128_pa
 
 def run_gemm_variants(dev, iters: int) -> dict:
     """mx_gemm_nt alone on the benchmark's products, cold operands (rotating copies), in the shipped tiling/schedule and in
-    the selectable alternatives: same product bit for bit, timed against each other."""
+    the three alternatives of the variants library (csrc/mx_gemm_variants.h): same product bit for bit, timed against each other."""
     import torch
 
     from kohakuwullm_amd import _lib
@@ -637,8 +637,9 @@ def run_gemm_variants(dev, iters: int) -> dict:
             def call():
                 aq, sa, bq, sb = ops[state["i"] % copies]
                 state["i"] += 1
-                _lib.invoke("mx_gemm_nt", 0, aq, aq.data_ptr(), sa.data_ptr(), bq.data_ptr(), sb.data_ptr(), c.data_ptr(), 0,
-                            m, n, k, k, k // 32, k, k // 32, n, flag, ws.data_ptr(), ws.numel())
+                fn = (_lib.load_variants() if flag else _lib.load()).mx_gemm_nt
+                _lib.check(fn(aq.data_ptr(), sa.data_ptr(), bq.data_ptr(), sb.data_ptr(), c.data_ptr(), 0, m, n, k, k, k // 32,
+                              k, k // 32, n, flag, ws.data_ptr(), ws.numel(), _lib.stream_of(aq)), "mx_gemm_nt")
 
             ts = _event_times(call, iters, warm=copies)
             state["i"] = 0
@@ -669,7 +670,7 @@ def standalone_line(args, dev) -> dict:
         return {"metric": "MXFP8 GEMM TFLOP/s (mx_gemm_nt alone, cold operands, shipped tiling)", "value": round(val, 1), "unit": "TFLOP/s",
                 "ms_per_step": round(secs * 1e3, 4), "dtype": "e4m3 x e4m3, ue8m0 scales, fp32 accumulate, bf16 out", **common,
                 "config": {"workload": "the six products of BASELINE configs[1] and the 8192^3 of configs[4], each alone; the shipped 256x256 "
-                                       "lockstep kernel against MX_EPI_PHASED and MX_EPI_TILE_128", **res},
+                                       "lockstep kernel of the product library against the three kernels of the variants library", **res},
                 "roofline": {"kernel": "gemm_nt_kernel", "bound": "mfma", "achieved": round(val, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(val / MFMA_PEAK_TFLOPS, 4), "traffic": None, "peak_measured": peaks["mfma_tflops"],
                              "frac_of_measured": round(val / peaks["mfma_tflops"], 4)}}
@@ -716,11 +717,13 @@ def main() -> None:
                          "measured bandwidth and MFMA rate")
     ap.add_argument("--routing", default="draws", choices=("draws", "ranked"),
                     help="moe: per-expert loads drawn i.i.d. Zipf (six full experts with the fixed seed) or Zipf by rank (59 live experts)")
-    ap.add_argument("--samples", type=int, default=0,
+    ap.add_argument("--samples", type=int, default=100,
                     help="after the timed region, time this many further steps one by one (events around each) and report "
-                         "their median and best; 100 or more for a publishable distribution")
+                         "their median and best beside the K-step mean (the reference's protocol, bench/core/timing.py:35-63: "
+                         "100 or more samples, median and best); 0 switches it off")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--breakdown", action="store_true", help="per-entry-point launch times of one step, on stderr")
+    ap.add_argument("--breakdown", action="store_true",
+                    help="also print the per-entry-point launch times of a step (the line's launch_breakdown) on stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, run one device copy of 256 MiB: a kernel of known traffic "
                          "against which a counter run (FETCH_SIZE / WRITE_SIZE) is scaled")
@@ -768,6 +771,8 @@ def main() -> None:
 
         ts = _event_times(one, args.samples, warm=0)
         sampled = {"ms_per_step_median": round(ts[len(ts) // 2], 4), "ms_per_step_best": round(ts[0], 4), "samples": len(ts)}
+        if gflop:
+            sampled["value_at_median"] = round(gflop / ts[len(ts) // 2], 2)
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -782,14 +787,19 @@ def main() -> None:
         step(i)
     torch.cuda.synchronize()
     records, _lib.TIMER = _lib.TIMER, None
-    if args.breakdown:
-        per_step = len(records) // args.steps
-        for j in range(per_step):
-            ts = sorted(records[i * per_step + j][2].elapsed_time(records[i * per_step + j][3]) for i in range(args.steps))
-            name, work = records[j][0], records[j][1]
-            rate = work / (ts[len(ts) // 2] * 1e-3)
+    # per entry-point call of a step, in launch order: median device time over the steps and the rate it gives
+    launches = []
+    per_step = len(records) // args.steps if args.steps and len(records) % args.steps == 0 else 0
+    for j in range(per_step):
+        ts = sorted(records[i * per_step + j][2].elapsed_time(records[i * per_step + j][3]) for i in range(args.steps))
+        name, work = records[j][0], records[j][1]
+        rate = work / (ts[len(ts) // 2] * 1e-3)
+        is_gemm = name in GEMM_ENTRIES
+        launches.append({"entry": name, "us_median": round(ts[len(ts) // 2] * 1e3, 1), "us_best": round(ts[0] * 1e3, 1),
+                         "rate_median": round(rate / (1e12 if is_gemm else 1e9), 1), "unit": "TFLOP/s" if is_gemm else "GB/s"})
+        if args.breakdown:
             print(f"  {j:2d} {name:28s} median {ts[len(ts) // 2] * 1e3:8.1f} us   "
-                  + (f"{rate / 1e12:7.1f} TFLOP/s" if name in GEMM_ENTRIES else f"{rate / 1e9:7.0f} GB/s"), file=sys.stderr)
+                  + (f"{rate / 1e12:7.1f} TFLOP/s" if is_gemm else f"{rate / 1e9:7.0f} GB/s"), file=sys.stderr)
     gemm = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n in GEMM_ENTRIES]
     quant = [(n, w, a.elapsed_time(b)) for n, w, a, b in records if n not in GEMM_ENTRIES]
     gemm_flops, gemm_ms = sum(w for _, w, _ in gemm), sum(t for _, _, t in gemm)
@@ -819,7 +829,7 @@ def main() -> None:
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(quant_gbs / HBM_PEAK_GBS, 4), "traffic": None,
                          "peak_measured": stream_peak, "frac_of_measured": round(quant_gbs / stream_peak, 4),
                          "launches": len(quant), "avg_launch_us": round(quant_ms / len(quant) * 1e3, 2)},
-            **sampled, **extra,
+            **sampled, **extra, "launch_breakdown": launches,
         }))
         return
     gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
@@ -875,6 +885,7 @@ def main() -> None:
         },
         "peaks_measured": peaks,
         "weight_refresh_ms": round(weight_refresh_ms, 4),
+        "launch_breakdown": launches,
     }
     if not args.no_cpu_baseline and args.workload == "ffn":
         out["cpu_baseline"] = cpu_baseline(device_rows=step.sample_rows())

@@ -51,17 +51,7 @@ enum mx_epilogue {
     MX_EPI_NONE = 0,      /* C = A B^T, cast to c_dtype */
     MX_EPI_ACCUMULATE = 1 /* C += A B^T with fp32 atomic adds; c_dtype must be MX_FP32 */
 };
-/* OR into `epilogue` of mx_gemm_nt: run on 128 x 128 tiles with two workgroups per compute unit instead of one
- * 256 x 256 tile (same product; a tiling choice kept selectable so the two can be timed against each other). */
-#define MX_EPI_TILE_128 0x10
-/* OR into `epilogue` of mx_gemm_nt: the 256 x 256 tile with its eight waves as two groups of four half a K stage
- * apart (two barriers per stage) instead of all eight in lockstep.  Same product bit for bit; selectable so the
- * two schedules can be timed against each other. */
-#define MX_EPI_PHASED 0x20
-/* OR into `epilogue` of mx_gemm_nt: the 256 x 256 tile on four waves, one per SIMD, 128 x 128 each, accumulators in
- * the accumulation registers and the next stage's first operands read under the current stage's last MFMAs.  Same
- * product bit for bit; selectable so the schedules can be timed against each other. */
-#define MX_EPI_WIDE_WAVES 0x40
+/* Bits 4-7 of `epilogue` select nothing in this library: mx_gemm_nt answers MX_EUNSUPPORTED when one is set. */
 /* OR into `epilogue` to cut K into n slices that run as independent tiles (needs
  * MX_EPI_ACCUMULATE and a caller-zeroed C): fills the GPU when M*N alone gives too few tiles. */
 #define MX_EPI_SPLIT_K(n) ((n) << 8)
@@ -228,6 +218,8 @@ int mx_unswizzle_scales(const uint8_t *swizzled, int64_t rows, int64_t cols, uin
  * workspace, a second kernel adds them in a fixed order).  With less, every tile is computed
  * whole: same product, fp32 sums in another order, slower on such shapes.  The workspace holds
  * nothing between calls; calls that may overlap in time need separate ones.
+ * epilogue: MX_EPI_NONE, or MX_EPI_ACCUMULATE optionally with MX_EPI_SPLIT_K(n); a negative value is
+ * MX_EINVAL, any other bit of the low byte MX_EUNSUPPORTED.
  * Replaces mxfp8_matmul_pq / _mxfp8_matmul_pq
  * (src/kohakuwullm/kernels/mxfp8/quantize.py:242-371) and the cuBLAS route
  * mxfp8_mm_swizzled (src/kohakuwullm/kernels/mxfp8/interop.py:51-122); the reference's
@@ -489,7 +481,8 @@ int mx_ubench_stream(int kind, const void *a, const void *b, void *c, int64_t ou
 /*
  * Register-resident loop of the block-scaled fp8 MFMA (bit 0 of wide clear: v_mfma_scale_f32_16x16x128_f8f6f4
  * with 8 independent accumulator tiles per wave, set: ..._32x32x64_... with 4), 8 waves on every CU (bit 1 of
- * wide set: 4 waves, one per SIMD), `iters` rounds; operands zero or (random != 0) a per-lane hash.  Returns the number of MFMA
+ * wide set: 4 waves, one per SIMD; bit 2 set, 16x16x128 form only: scale bytes come from vector registers instead
+ * of an inline constant), `iters` rounds; operands zero or (random != 0) a per-lane hash.  Returns the number of MFMA
  * instructions the launch issues (each 2 * 16*16*128 = 65536 or 2 * 32*32*64 = 131072 FLOP) or a
  * negative mx_status.  out: one float per launched thread (512 x CUs).  The reference's rule for a
  * compute ceiling: measured from registers with independent accumulators

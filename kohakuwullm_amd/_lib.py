@@ -117,6 +117,26 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+# The dense GEMM's three measured-slower alternative kernels live in a library of their own, built from the same
+# sources with -DMX_BENCH_VARIANTS (csrc/mx_gemm_variants.h); only the GEMM benchmark and the bit-equality test of
+# the kernels load it.  The flags are theirs: the product library answers MX_EUNSUPPORTED to each.
+VARIANTS_PATH = os.path.join(_HERE, "libmxfp8_hip_variants.so")
+MX_EPI_TILE_128, MX_EPI_PHASED, MX_EPI_WIDE_WAVES = 0x10, 0x20, 0x40
+_variants: ctypes.CDLL | None = None
+
+
+def load_variants() -> ctypes.CDLL:
+    """The variants library with ``mx_gemm_nt`` typed (every other entry point is the product library's)."""
+    global _variants
+    if _variants is None:
+        if not os.path.exists(VARIANTS_PATH):
+            raise MXFP8LibraryError(f"{VARIANTS_PATH} is missing: `make -C {os.path.join(_HERE, 'csrc')}` builds it")
+        lib = ctypes.CDLL(VARIANTS_PATH)
+        lib.mx_gemm_nt.restype, lib.mx_gemm_nt.argtypes = SIGNATURES["mx_gemm_nt"]
+        _variants = lib
+    return _variants
+
+
 def check(status: int, what: str) -> None:
     if status == MX_OK:
         return
@@ -135,20 +155,25 @@ def stream_of(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-_WORKSPACE_BYTES: dict[int, int] = {}
+_WORKSPACES: dict[tuple[int, int], torch.Tensor] = {}
 
 
 def gemm_workspace(t: torch.Tensor) -> torch.Tensor:
     """Scratch for the K splits of ``mx_gemm_nt`` / ``mx_gemm_nt_batch`` / ``mx_grouped_wgrad_nt`` on ``t``'s device.
 
-    It comes from PyTorch's caching allocator on the current stream, per call: the block is reused by the
-    next call on that stream and is never touched by work on another one.  The library itself allocates nothing.
+    One tensor per (device, current stream), allocated the first time that stream asks and kept: calls on one
+    stream run in order and may share it, work on another stream gets its own, and the hot path never goes
+    back to the allocator for a 128 MiB block that smaller tensors may have carved up in the meantime.
+    The library itself allocates nothing.
     """
     index = t.device.index if t.device.index is not None else torch.cuda.current_device()
-    if index not in _WORKSPACE_BYTES:
+    key = (index, stream_of(t))
+    ws = _WORKSPACES.get(key)
+    if ws is None:
         with torch.cuda.device(index):
-            _WORKSPACE_BYTES[index] = int(load().mx_gemm_workspace_bytes())
-    return torch.empty(_WORKSPACE_BYTES[index], dtype=torch.uint8, device=t.device)
+            ws = torch.empty(int(load().mx_gemm_workspace_bytes()), dtype=torch.uint8, device=t.device)
+        _WORKSPACES[key] = ws
+    return ws
 
 
 def require_gpu(t: torch.Tensor, name: str) -> None:

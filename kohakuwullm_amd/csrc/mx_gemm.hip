@@ -6,6 +6,9 @@
 #include <atomic>
 
 #include "mx_gemm_core.h"
+#ifdef MX_BENCH_VARIANTS
+#include "mx_gemm_variants.h"
+#endif
 
 namespace mx {
 
@@ -122,7 +125,7 @@ struct DenseProblem {
             int row = dma_row<S>(L, q);
             int chunk = (L.lane & 7) ^ swz_a(row);
             int grow = row < mrem ? row : mrem - 1;  // rows past M re-read the last row; never stored
-            c.a_voff[q] = (uint32_t)(grow * p.lda) + chunk * 16;
+            c.a_voff[q] = (uint32_t)(grow * p.lda) + chunk * 16 + copy_bias(q);
         }
 #pragma unroll
         for (int q = 0; q < S::QB; q++) {
@@ -130,12 +133,13 @@ struct DenseProblem {
             int chunk = (L.lane & 7) ^ swz_a(row);
             int brow = b_row_of_lds<S>(row);
             int grow = brow < nrem ? brow : nrem - 1;
-            c.b_voff[q] = (uint32_t)(grow * p.ldb) + chunk * 16;
+            c.b_voff[q] = (uint32_t)(grow * p.ldb) + chunk * 16 + copy_bias(q);
         }
         c.srow0 = scale_row(t, L.tid < S::BM + S::BN ? L.tid : 0);
         c.srow1 = S::TWO_ROWS ? scale_row(t, L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
     }
 
+#ifdef MX_BENCH_VARIANTS
     // the phased schedule's description of a tile: bases, pitches and limits; the lanes rebuild their offsets from them
     __device__ __forceinline__ void context(const Tile &t, const Lane &L0, PhasedCtx<S> &c) const {
         const Lane L = opaque(L0);
@@ -155,8 +159,10 @@ struct DenseProblem {
         c.srow0 = scale_row(t, L.tid);
         c.srow1 = nullptr;
     }
+#endif
 
-    static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
+    // stores an interior tile issues per lane: one per (i, v), two when a lane's run is 8 fp32 values (32 bytes)
+    static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 && S::NT == 8 ? 2 : 1);
     static constexpr bool EARLY_WAIT = false;  // interior tiles leave exactly NST stores in flight instead
 
     // Slot of workgroup `wg`'s piece of the split tile whose stages start at `begin` in the
@@ -228,6 +234,7 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
     persistent_gemm<S, K512>(prob, smem);
 }
 
+#ifdef MX_BENCH_VARIANTS
 // The same tiles under the phased schedule (two groups of four waves half a K stage apart): MX_EPI_PHASED.
 template <typename S, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_phased_kernel(DenseArgs args) {
@@ -253,6 +260,7 @@ __global__ __launch_bounds__(S::NTHR) __attribute__((amdgpu_waves_per_eu(2, 2)))
     DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
     persistent_gemm<S, K512>(prob, smem);
 }
+#endif
 
 // Several independent products in one launch.  The XCDs are partitioned among the problems
 // (x_lo[j] .. x_lo[j+1]) in proportion to their work, so a product with too few
@@ -475,6 +483,7 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
     dim3 grid((unsigned)(work < cus && !a.sk_tiles ? work : cus)), block(S::NTHR);
     int rc;
     a.phased = phased ? 1 : 0;
+#ifdef MX_BENCH_VARIANTS
     if constexpr (S::NW == 4)
         rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_wide_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
              : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_wide_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
@@ -484,6 +493,7 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
              : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
                                     : launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
     else
+#endif
         rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
              : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
                                     : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
@@ -495,6 +505,7 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
 
 // 256 x 256 x 128 tile, 8 waves as 4 (M) x 2 (N): a wave owns 64 x 128, a lane 8 consecutive N.
 typedef GemmShape<256, 256, 4, 2> DenseShape;
+#ifdef MX_BENCH_VARIANTS
 // 128 x 128 x 128 tile, 4 waves as 2 x 2: a wave owns 64 x 64, a lane 4 consecutive N; 73 KiB of LDS, two per CU.
 typedef GemmShape<128, 128, 2, 2> PairShape;
 // 256 x 256 x 128 tile, 4 waves as 2 x 2, one per SIMD: a wave owns 128 x 128 (the wide-wave schedule).
@@ -517,6 +528,7 @@ static int launch_pair(DenseArgs a, hipStream_t st) {
     if (rc != MX_OK) return rc;
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
+#endif
 
 static bool tiled_ok(const DenseArgs &a) {
     const int64_t M = a.M, N = a.N;
@@ -529,8 +541,12 @@ template <int CDT>
 static int gemm_dispatch(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bool pair = false, bool phased = false,
                          bool wide = false) {
     const int64_t M = a.M, N = a.N;
+#ifdef MX_BENCH_VARIANTS
     if (pair && tiled_ok(a) && a.split_k == 1 && !a.slice_ws) return launch_pair<CDT>(a, st);
     if (wide && tiled_ok(a)) return launch_tiled<WideShape, CDT>(a, ws, ws_slots, st, false);
+#else
+    if (pair || phased || wide) return MX_EUNSUPPORTED;
+#endif
     if (!tiled_ok(a)) {
         if (a.accumulate || a.a_ks || a.b_ks) return MX_EUNSUPPORTED;  // the element-wise kernel reads row-major only
         int64_t blocks = (M * N + 255) / 256;
@@ -766,11 +782,20 @@ extern "C" int mx_gemm_nt(const uint8_t *aq, const uint8_t *as, const uint8_t *b
     DenseArgs a;
     int rc = fill_args(a, aq, as, bq, bs, c, M, N, K, lda, ldas, ldb, ldbs, ldc);
     if (rc != MX_OK) return rc;
+    if (epilogue < 0) return MX_EINVAL;
     const int split_k = epilogue >> 8;  // MX_EPI_SPLIT_K(n)
-    const bool pair = (epilogue & MX_EPI_TILE_128) != 0, phased = (epilogue & MX_EPI_PHASED) != 0;
-    const bool wide = (epilogue & MX_EPI_WIDE_WAVES) != 0;
     const int epi = epilogue & 0x0F;
     if (epi != MX_EPI_NONE && epi != MX_EPI_ACCUMULATE) return MX_EUNSUPPORTED;
+#ifdef MX_BENCH_VARIANTS
+    const bool pair = (epilogue & MX_EPI_TILE_128) != 0, phased = (epilogue & MX_EPI_PHASED) != 0;
+    const bool wide = (epilogue & MX_EPI_WIDE_WAVES) != 0;
+    // one alternative kernel at a time, on a plain product: no unknown bit, no accumulation, no caller-driven K slices
+    if ((epilogue & 0x80) || (int)pair + (int)phased + (int)wide > 1) return MX_EUNSUPPORTED;
+    if ((pair || phased || wide) && (epi != MX_EPI_NONE || split_k > 1)) return MX_EUNSUPPORTED;
+#else
+    const bool pair = false, phased = false, wide = false;
+    if (epilogue & 0xF0) return MX_EUNSUPPORTED;  // bits 4-7 select nothing in this library
+#endif
     if (epi == MX_EPI_ACCUMULATE && c_dtype != MX_FP32) return MX_EINVAL;
     if (split_k > 1 && epi != MX_EPI_ACCUMULATE) return MX_EINVAL;
     if (c_dtype != MX_BF16 && c_dtype != MX_FP16 && c_dtype != MX_FP32) return MX_EINVAL;

@@ -334,12 +334,12 @@ struct GroupedProblem {
 #pragma unroll
         for (int q = 0; q < S::QA; q++) {
             const int row = dma_row<S>(L, q);
-            c.a_voff[q] = (uint32_t)((int64_t)a_src_row(t, row) * p.ldx) + (((L.lane & 7) ^ swz_a(row)) << 4);
+            c.a_voff[q] = (uint32_t)((int64_t)a_src_row(t, row) * p.ldx) + (((L.lane & 7) ^ swz_a(row)) << 4) + copy_bias(q);
         }
 #pragma unroll
         for (int q = 0; q < S::QB; q++) {
             const int row = dma_row<S>(L, q);
-            c.b_voff[q] = (uint32_t)((int64_t)b_src_row(t, row) * p.ldw) + (((L.lane & 7) ^ swz_a(row)) << 4);
+            c.b_voff[q] = (uint32_t)((int64_t)b_src_row(t, row) * p.ldw) + (((L.lane & 7) ^ swz_a(row)) << 4) + copy_bias(q);
         }
         auto srow = [&](int r) -> const uint8_t * {
             if (r < S::BM) return p.xs + (int64_t)a_src_row(t, r) * p.ldxs;
@@ -1006,13 +1006,13 @@ struct WgradProblem {
 #pragma unroll
         for (int q = 0; q < S::QA; q++) {
             const int row = dma_row<S>(L, q);
-            c.a_voff[q] = (uint32_t)((int64_t)(row < mrem ? row : mrem - 1) * p.lda) + (((L.lane & 7) ^ swz_a(row)) << 4);
+            c.a_voff[q] = (uint32_t)((int64_t)(row < mrem ? row : mrem - 1) * p.lda) + (((L.lane & 7) ^ swz_a(row)) << 4) + copy_bias(q);
         }
 #pragma unroll
         for (int q = 0; q < S::QB; q++) {
             const int row = dma_row<S>(L, q);
             const int brow = b_row_of_lds<S>(row);
-            c.b_voff[q] = (uint32_t)((int64_t)(brow < nrem ? brow : nrem - 1) * p.ldb) + (((L.lane & 7) ^ swz_a(row)) << 4);
+            c.b_voff[q] = (uint32_t)((int64_t)(brow < nrem ? brow : nrem - 1) * p.ldb) + (((L.lane & 7) ^ swz_a(row)) << 4) + copy_bias(q);
         }
         auto srow = [&](int r) -> const uint8_t * {
             if (r < S::BM) return p.as + (int64_t)(t.m0 + (r < mrem ? r : mrem - 1)) * p.ldas;

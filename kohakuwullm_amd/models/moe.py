@@ -281,7 +281,7 @@ class MoEMLP(nn.Module):
         offsets, order, token_of, _ = expert_sort(topk_idx.reshape(-1), counts, topk_idx.shape[-1], self.num_buckets)
         out = self._routed(flat, topk_weight, order, token_of, offsets)
         if self.shared is not None:
-            out = out + self.shared(flat).to(out.dtype)
+            out = out + self.shared(flat)  # dtype by promotion, as the reference's forward (components/moe.py:395-449)
         return out.reshape(shape)
 
     def router_losses(self) -> torch.Tensor | None:

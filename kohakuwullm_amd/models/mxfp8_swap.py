@@ -9,7 +9,8 @@ converted with ``enable_mxfp8()``; anything matmul-shaped that nobody claimed bl
 
 Where the reference selects parents by class, this swap selects by the attribute names
 alone, so it works on the reference's module classes and on this package's without
-importing either.  ``kohakuwullm_amd.MXFP8Linear`` is equally valid as the ``linear_cls``
+importing either -- and converts an ``nn.Linear`` called ``up``, ``fc1``, ... under ANY parent,
+which the reference would leave alone; pass ``scope`` to keep it to the blocks that are meant.  ``kohakuwullm_amd.MXFP8Linear`` is equally valid as the ``linear_cls``
 argument of the reference's own ``swap_mxfp8``.
 """
 
@@ -168,6 +169,12 @@ def _declarations(parent: nn.Module) -> dict[str, Matmul]:
     said: dict[str, Matmul] = {}
     if isinstance(parent, nn.Embedding):
         said["weight"] = Matmul(0, "an embedding is a gather, not a GEMM", never=True)
+    # The LM head (src/kohakuwullm/models/mxfp8_swap.py:133-139 names its class; here: a module whose class is called
+    # LMHead and that holds a bare (vocab, dim) ``projection``) stays 16-bit by design.
+    projection = getattr(parent, "projection", None)
+    if type(parent).__name__ == "LMHead" and isinstance(projection, nn.Parameter) and projection.dim() == 2:
+        vocab, dim = projection.shape
+        said["projection"] = Matmul(vocab * dim, "the head contracts over the vocabulary", never=True)
     declare = getattr(parent, DECLARE, None)
     if callable(declare):
         said.update(declare())

@@ -375,7 +375,7 @@ def test_workspace_is_the_callers(oracle, m, n, k):
 def test_tilings_and_schedules_agree(oracle, m, n, k):
     """The 256 x 256 tile in lockstep (default), the same tile with its waves in two groups half a stage apart
     (MX_EPI_PHASED), 128 x 128 tiles with two workgroups per CU (MX_EPI_TILE_128) and the 256 x 256 tile on four
-    waves of 128 x 128 (MX_EPI_WIDE_WAVES): every element contracts the same K sequence whichever computes it, so
+    waves of 128 x 128 (MX_EPI_WIDE_WAVES) -- the three alternatives of the variants library: every element contracts the same K sequence whichever computes it, so
     all four agree bit for bit; held to the oracle on sampled rows (the last rows, in a ragged tile, among them).
     With a workspace the default, the phased and the wide-wave schedule may also split K the same way: equal again."""
     from kohakuwullm_amd import _lib
@@ -385,12 +385,23 @@ def test_tilings_and_schedules_agree(oracle, m, n, k):
     a, sa, b, sb = aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)
     ws = _lib.gemm_workspace(a)
 
+    variants = _lib.load_variants()  # the shipped kernel (flag 0) is run from the product library
+
     def run(epilogue, dtype=torch.bfloat16, workspace=None):
         c = torch.full((m, n), float("nan"), device=DEV, dtype=dtype)
-        _lib.invoke("mx_gemm_nt", 0, a, a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(),
-                    _lib.MX_DTYPE[dtype], m, n, k, k, k // 32, k, k // 32, n, epilogue,
-                    None if workspace is None else workspace.data_ptr(), 0 if workspace is None else workspace.numel())
+        fn = variants.mx_gemm_nt if epilogue else _lib.load().mx_gemm_nt
+        _lib.check(fn(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(), _lib.MX_DTYPE[dtype], m, n, k,
+                      k, k // 32, k, k // 32, n, epilogue, None if workspace is None else workspace.data_ptr(),
+                      0 if workspace is None else workspace.numel(), _lib.stream_of(a)), "mx_gemm_nt")
         return c
+
+    # the product library has none of the alternatives and says so
+    for flag in (0x10, 0x20, 0x40, 0x80, 0x30):
+        c = torch.empty(m, n, device=DEV, dtype=torch.bfloat16)
+        assert _lib.load().mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(), 0, m, n, k, k,
+                                      k // 32, k, k // 32, n, flag, None, 0, _lib.stream_of(a)) == _lib.MX_EUNSUPPORTED
+    assert variants.mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), c.data_ptr(), 0, m, n, k, k,
+                               k // 32, k, k // 32, n, 0x30, None, 0, _lib.stream_of(a)) == _lib.MX_EUNSUPPORTED  # two at once
 
     default, phased, small, wide = run(0), run(0x20), run(0x10), run(0x40)  # MX_EPI_PHASED, MX_EPI_TILE_128, MX_EPI_WIDE_WAVES
     assert torch.isfinite(default.float()).all()

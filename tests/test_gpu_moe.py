@@ -576,6 +576,11 @@ def test_moe_module_reference_defaults(oracle):
     route_on = torch.randn(200, 256, device=DEV)
     with torch.autocast("cuda", dtype=torch.bfloat16):
         assert not torch.equal(moe(x, route_on=route_on), moe(x))
+    # fp32 activations outside autocast: the routed MXFP8 path answers in bf16, a 16-bit shared expert (fp32 weights,
+    # never swapped) in fp32, and their sum takes the promoted dtype, as in the reference's forward
+    plain = MoEMLP(256, hidden=128, num_experts=16, top_k=4).to(DEV)
+    plain.enable_mxfp8()
+    assert plain(x).dtype == torch.float32
     # the per-expert loop is the eager test arm: the swap refuses it and says why
     loop = MoEMLP(256, hidden=128, num_experts=4, top_k=2, num_shared=0, dense_fallback=True).to(DEV)
     rep = swap_mxfp8(loop)

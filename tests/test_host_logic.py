@@ -109,6 +109,34 @@ def test_swap_accounting_on_cpu():
     assert {"ok.w", "unreached.w"} <= {n for n, _ in r3.unreached}
 
 
+def test_swap_leaves_the_lm_head_alone():
+    """A backbone with an LM head (a bare (vocab, dim) ``projection`` on a module whose class is called LMHead, as the
+    reference's): the head is 16-bit by design, charged to `never`, and does not block the swap."""
+    from kohakuwullm_amd.models.mlp import SwiGLU
+    from kohakuwullm_amd.models.mxfp8_swap import swap_mxfp8
+
+    class LMHead(nn.Module):
+        def __init__(self, vocab, dim):
+            super().__init__()
+            self.projection = nn.Parameter(torch.zeros(vocab, dim))
+
+    class NotAHead(nn.Module):  # the same tensor under another class name is nobody's: it blocks
+        def __init__(self):
+            super().__init__()
+            self.projection = nn.Parameter(torch.zeros(5, 128))
+
+    class Backbone(nn.Module):
+        def __init__(self, head):
+            super().__init__()
+            self.mlp = SwiGLU(128, hidden=256)
+            self.head = head
+
+    report = swap_mxfp8(Backbone(LMHead(1000, 128)), linear_cls=_StubLinear)
+    assert not report.blocking and report.by_design == ["head.projection"] and report.mac["never"] == 1000 * 128
+    other = swap_mxfp8(Backbone(NotAHead()), linear_cls=_StubLinear)
+    assert other.blocking and other.unaccounted == ["head.projection(5, 128)"]
+
+
 def test_module_contracts_without_gpu():
     from kohakuwullm_amd._lib import MXFP8LibraryError
     from kohakuwullm_amd.kernels.mxfp8 import mxfp8_matmul_pq, quantize_mx
