@@ -246,23 +246,43 @@ def _event_times(fn, iters: int, warm: int = 3):
     return sorted(a.elapsed_time(b) for a, b in pairs)
 
 
-def measure_stream(dev, out_bytes: int = 1 << 30, iters: int = 10) -> dict:
-    """Streaming bandwidth of this device in GB/s (best and median of `iters` launches on 1 GiB per operand):
-    read, copy, triad, and a 2-bytes-read-per-byte-written mix (the traffic of a 16-bit -> 8-bit cast)."""
+STREAM_KINDS = (("read", 0, 1), ("copy", 1, 2), ("triad", 2, 3), ("read2_write1", 3, 3), ("read2_write1_two_streams", 4, 3),
+                ("read3_write2", 5, 5))  # name, kind of mx_ubench_stream_cfg, bytes moved per output byte
+# launch shapes swept per mix: (threads, unroll, workgroups per CU [0: one chunk each], non-temporal bits [1 loads, 2 stores])
+STREAM_SWEEP_FULL = tuple((t, u, w, nt) for t in (256, 512, 1024) for u in (2, 4, 8) for w in (0, 8, 16, 32) for nt in (0, 1, 2, 3))
+STREAM_SWEEP_SHORT = tuple((t, u, w, nt) for t in (256, 512) for u in (4, 8) for w in (0, 16) for nt in (0, 3))
+STREAM_DEFAULT_POINT = (256, 4, 16, 3)  # what mx_ubench_stream runs
+
+
+def measure_stream(dev, out_bytes: int = 1 << 29, iters: int = 10, sweep=STREAM_SWEEP_SHORT) -> dict:
+    """Streaming bandwidth of this device in GB/s per traffic mix: read, copy, triad, the 2 : 1 mix of a 16-bit -> 8-bit
+    cast (from one and from two input streams) and the 3 : 2 mix of the SwiGLU' quantizer.  Every mix is run under every
+    launch shape of `sweep` (best of 3 launches each), then `iters` more launches of the best shape give best and
+    median; `fixed_point` is the one shape mx_ubench_stream itself runs.  A ceiling is the best of the sweep: a product
+    kernel that beats it says the sweep is too narrow."""
     import torch
 
     from kohakuwullm_amd import _lib
 
     lib = _lib.load()
-    a = torch.empty(2 * out_bytes, dtype=torch.uint8, device=dev).random_(0, 255)  # kind 3 reads twice what it writes
+    a = torch.empty(3 * out_bytes, dtype=torch.uint8, device=dev).random_(0, 255)  # kind 5 reads three streams
     b = torch.empty(out_bytes, dtype=torch.uint8, device=dev).random_(0, 255)
-    c = torch.empty(out_bytes, dtype=torch.uint8, device=dev)
+    c = torch.empty(2 * out_bytes, dtype=torch.uint8, device=dev)                  # ... and writes two
     st = torch.cuda.current_stream(dev).cuda_stream
     out = {}
-    for name, kind, moved in (("read", 0, out_bytes), ("copy", 1, 2 * out_bytes), ("triad", 2, 3 * out_bytes), ("read2_write1", 3, 3 * out_bytes)):
-        ts = _event_times(lambda: _lib.check(lib.mx_ubench_stream(kind, a.data_ptr(), b.data_ptr(), c.data_ptr(), out_bytes, st),
-                                             "mx_ubench_stream"), iters)
-        out[name] = {"best": round(moved / ts[0] / 1e6, 1), "median": round(moved / ts[len(ts) // 2] / 1e6, 1)}
+
+    def timed(kind, shape, n):
+        t, u, w, nt = shape
+        return _event_times(lambda: _lib.check(lib.mx_ubench_stream_cfg(kind, t, u, w, nt, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+                                                                        out_bytes, st), "mx_ubench_stream_cfg"), n, warm=1)
+
+    for name, kind, factor in STREAM_KINDS:
+        moved = factor * out_bytes
+        best_shape = min(sweep, key=lambda shape: timed(kind, shape, 3)[0])
+        ts, fixed = timed(kind, best_shape, iters), timed(kind, STREAM_DEFAULT_POINT, 3)
+        out[name] = {"best": round(moved / ts[0] / 1e6, 1), "median": round(moved / ts[len(ts) // 2] / 1e6, 1),
+                     "shape": dict(zip(("threads", "unroll", "wgs_per_cu", "nontemporal"), best_shape)),
+                     "fixed_point": round(moved / fixed[0] / 1e6, 1)}
     del a, b, c
     return out
 
@@ -326,17 +346,20 @@ def measured_peaks(dev) -> dict:
     MFMA loop on hashed operands (TFLOP/s), in single launches from an idle clock and sustained; the kernels are
     priced against the larger of the two (zero operands clock higher still and are reported by --workload peak)."""
     stream, mfma = measure_stream(dev, iters=5), measure_mfma(dev, iters=2000, repeats=3)
+    two_to_one = max(stream["read2_write1"]["best"], stream["read2_write1_two_streams"]["best"])
     short = max(v["best"] for k, v in mfma.items() if k.endswith("hashed"))
     sustained = measure_mfma_sustained(dev)
     return {
         "hbm_gbs": max(v["best"] for v in stream.values()),
-        "hbm_read2_write1_gbs": stream["read2_write1"]["best"],
+        "hbm_read2_write1_gbs": two_to_one,
+        "hbm_read3_write2_gbs": stream["read3_write2"]["best"],
         "hbm_copy_gbs": stream["copy"]["best"],
         "mfma_tflops": max(short, sustained),
         "mfma_tflops_single_launch": short,
         "mfma_tflops_sustained": sustained,
-        "how": "mx_ubench_stream on 1 GiB per operand, best of a few launches; mx_ubench_mfma from registers, best single "
-               "launch and the last 60 of 240 back-to-back launches; all in this run",
+        "how": "mx_ubench_stream_cfg on 512 MiB per stream, every mix under 16 launch shapes (threads, loads in flight, grid, "
+               "non-temporal hints), best launch of the best shape; mx_ubench_mfma from registers, best single launch and the "
+               "last 60 of 240 back-to-back launches; all in this run",
     }
 
 # Bytes the GEMM launches of one step move between the L2s and the fabric, per launch, from the
@@ -675,11 +698,13 @@ def standalone_line(args, dev) -> dict:
                              "frac": round(val / MFMA_PEAK_TFLOPS, 4), "traffic": None, "peak_measured": peaks["mfma_tflops"],
                              "frac_of_measured": round(val / peaks["mfma_tflops"], 4)}}
     if args.workload == "stream":
-        bw = measure_stream(dev, iters=max(args.steps, 10))
+        bw = measure_stream(dev, iters=max(args.steps, 10), sweep=STREAM_SWEEP_FULL)
         best = max(v["best"] for v in bw.values())
-        return {"metric": "device streaming bandwidth GB/s (best of read / copy / triad / 2:1 mix)", "value": best, "unit": "GB/s",
+        return {"metric": "device streaming bandwidth GB/s (best of read / copy / triad / 2:1 / 3:2 mixes)", "value": best, "unit": "GB/s",
                 "ms_per_step": None, "dtype": "bytes", **common,
-                "config": {"workload": "1 GiB per operand, non-temporal 16-byte accesses, grid-stride (mx_ubench_stream)", "patterns": bw},
+                "config": {"workload": f"512 MiB per stream, 16-byte accesses, every mix under {len(STREAM_SWEEP_FULL)} launch shapes "
+                                       "(threads 256-1024, 2-8 accesses in flight, one chunk per workgroup or 8-32 workgroups per CU, "
+                                       "temporal or non-temporal loads and stores): mx_ubench_stream_cfg", "patterns": bw},
                 "roofline": {"kernel": "stream_kernel", "bound": "hbm", "achieved": best, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": round(best / HBM_PEAK_GBS, 4), "traffic": None}}
     if args.workload == "peak":
@@ -721,6 +746,9 @@ def main() -> None:
                     help="after the timed region, time this many further steps one by one (events around each) and report "
                          "their median and best beside the K-step mean (the reference's protocol, bench/core/timing.py:35-63: "
                          "100 or more samples, median and best); 0 switches it off")
+    ap.add_argument("--variants-library", action="store_true",
+                    help="run the workload on libmxfp8_hip_variants.so instead of the product library: for moe, the two fused "
+                         "expert kernels on 128 x 128 tiles with two workgroups per CU (measured slower; kept as evidence)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true",
                     help="also print the per-entry-point launch times of a step (the line's launch_breakdown) on stderr")
@@ -736,6 +764,8 @@ def main() -> None:
     from kohakuwullm_amd import _lib
 
     dev = torch.device("cuda:0")
+    if args.variants_library:
+        _lib.variants_library().__enter__()  # for the rest of the process
     _lib.check(_lib.load().mx_device_supported(0), "mx_device_supported")
     if args.workload in ("quant", "gemm", "stream", "peak"):
         print(json.dumps(standalone_line(args, dev)))

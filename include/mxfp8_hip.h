@@ -479,6 +479,20 @@ int mx_combine_routed_backward(const void *grad_out, int64_t ldg, const void *ro
 int mx_ubench_stream(int kind, const void *a, const void *b, void *c, int64_t out_bytes, void *stream);
 
 /*
+ * The same streaming kernels with their launch shape as arguments, so that the ceiling a quantizer is priced against is
+ * the best of a sweep and not one fixed point: threads per workgroup (a multiple of 64, at most 1024), 16-byte accesses
+ * of every stream in flight per lane (unroll: 1, 2, 4 or 8), workgroups per compute unit of the grid-stride grid (0: one
+ * chunk per workgroup, no loop), nontemporal bit 0: loads carry the non-temporal hint, bit 1: stores do.  Two more
+ * traffic mixes beside kinds 0-3 of mx_ubench_stream: kind 4 reads a[i] and a[n + i] and writes c[i] (2 : 1 from two
+ * input streams; a holds 2 x out_bytes), kind 5 reads a[i], a[n + i], a[2n + i] and writes c[i], c[n + i] (3 : 2, the
+ * SwiGLU' quantizer's mix; a holds 3 x out_bytes, c 2 x out_bytes; n = out_bytes / 16).  mx_ubench_stream(kind, ...) is
+ * (256 threads, unroll 4, 16 workgroups per CU, both hints).  Same rule of the reference as above
+ * (src/kohakuwullm/bench/core/timing.py:231-268).
+ */
+int mx_ubench_stream_cfg(int kind, int threads, int unroll, int wgs_per_cu, int nontemporal, const void *a,
+                         const void *b, void *c, int64_t out_bytes, void *stream);
+
+/*
  * Register-resident loop of the block-scaled fp8 MFMA (bit 0 of wide clear: v_mfma_scale_f32_16x16x128_f8f6f4
  * with 8 independent accumulator tiles per wave, set: ..._32x32x64_... with 4), 8 waves on every CU (bit 1 of
  * wide set: 4 waves, one per SIMD; bit 2 set, 16x16x128 form only: scale bytes come from vector registers instead

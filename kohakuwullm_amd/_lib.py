@@ -70,6 +70,7 @@ SIGNATURES = {
     "mx_gemm_workspace_bytes": (_i64, []),
     "mx_gemm_nt_batch": (_ci, [_p, _ci, _ci, _p, _i64, _p]),
     "mx_ubench_stream": (_ci, [_ci, _p, _p, _p, _i64, _p]),
+    "mx_ubench_stream_cfg": (_ci, [_ci, _ci, _ci, _ci, _ci, _p, _p, _p, _i64, _p]),
     "mx_ubench_mfma": (_i64, [_ci, _ci, _ci, _p, _i64, _p]),
 }
 
@@ -117,24 +118,43 @@ def load() -> ctypes.CDLL:
     return lib
 
 
-# The dense GEMM's three measured-slower alternative kernels live in a library of their own, built from the same
-# sources with -DMX_BENCH_VARIANTS (csrc/mx_gemm_variants.h); only the GEMM benchmark and the bit-equality test of
-# the kernels load it.  The flags are theirs: the product library answers MX_EUNSUPPORTED to each.
+# Measured-slower alternative kernels live in a library of their own, built from the same sources with
+# -DMX_BENCH_VARIANTS: the dense GEMM's three other tilings / schedules behind flags of `epilogue`
+# (csrc/mx_gemm_variants.h; the product library answers MX_EUNSUPPORTED to each), and the two fused expert kernels on
+# 128 x 128 tiles with two workgroups per CU in place of the shipped 256 x 256 ones (csrc/mx_grouped.hip).  Only the
+# benchmark (--variants-library) and the bit-equality tests of the kernels load it.
 VARIANTS_PATH = os.path.join(_HERE, "libmxfp8_hip_variants.so")
 MX_EPI_TILE_128, MX_EPI_PHASED, MX_EPI_WIDE_WAVES = 0x10, 0x20, 0x40
 _variants: ctypes.CDLL | None = None
 
 
 def load_variants() -> ctypes.CDLL:
-    """The variants library with ``mx_gemm_nt`` typed (every other entry point is the product library's)."""
+    """The variants library, typed like the product library."""
     global _variants
     if _variants is None:
         if not os.path.exists(VARIANTS_PATH):
             raise MXFP8LibraryError(f"{VARIANTS_PATH} is missing: `make -C {os.path.join(_HERE, 'csrc')}` builds it")
         lib = ctypes.CDLL(VARIANTS_PATH)
-        lib.mx_gemm_nt.restype, lib.mx_gemm_nt.argtypes = SIGNATURES["mx_gemm_nt"]
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = restype, argtypes
         _variants = lib
     return _variants
+
+
+class variants_library:
+    """``with variants_library():`` every entry point called inside goes to the variants library (benchmarks and tests only)."""
+
+    def __enter__(self):
+        global _lib
+        load()
+        self._saved, _lib = _lib, load_variants()
+        return _lib
+
+    def __exit__(self, *exc):
+        global _lib
+        _lib = self._saved
+        return False
 
 
 def check(status: int, what: str) -> None:

@@ -61,6 +61,21 @@ __device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_
 template <int DT>
 struct Elem;
 
+// Bulk loads and stores of the streaming kernels, with or without the non-temporal hint.  The hint pays for data that is
+// read once or written for a consumer far away (measured inside a feed-forward step: the SwiGLU' quantizer 148 -> 131 us
+// with hinted loads) and costs where the next kernel would have found the lines in the last-level cache (codes of a 48 MB
+// activation written with the hint: the GEMM that reads them next 186 -> 191 us), so each kernel chooses.
+template <bool NT, typename V>
+__device__ __forceinline__ V stream_load(const V *p) {
+    if (NT) return __builtin_nontemporal_load(p);
+    return *p;
+}
+template <bool NT, typename V>
+__device__ __forceinline__ void stream_store(V *p, V v) {
+    if (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
 template <>
 struct Elem<MX_BF16> {
     typedef uint16_t type;
@@ -75,7 +90,8 @@ struct Elem<MX_BF16> {
     static __device__ __forceinline__ float load1(const void *p) { return bits2f((uint32_t)(*(const uint16_t *)p) << 16); }
     // The same load in two halves, so that a kernel can put many of them in flight before it converts any.
     typedef v4i raw;
-    static __device__ __forceinline__ raw load_raw(const void *p) { return *(const v4i *)p; }
+    template <bool NT = false>
+    static __device__ __forceinline__ raw load_raw(const void *p) { return stream_load<NT>((const v4i *)p); }
     static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -96,7 +112,8 @@ struct Elem<MX_FP16> {
     }
     static __device__ __forceinline__ float load1(const void *p) { return (float)(*(const _Float16 *)p); }
     typedef _Float16 raw __attribute__((ext_vector_type(8)));
-    static __device__ __forceinline__ raw load_raw(const void *p) { return *(const raw *)p; }
+    template <bool NT = false>
+    static __device__ __forceinline__ raw load_raw(const void *p) { return stream_load<NT>((const raw *)p); }
     static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
 #pragma unroll
         for (int i = 0; i < 8; i++) v[i] = (float)r[i];
@@ -118,7 +135,10 @@ struct Elem<MX_FP32> {
     struct raw {
         v4f a, b;
     };
-    static __device__ __forceinline__ raw load_raw(const void *p) { return raw{((const v4f *)p)[0], ((const v4f *)p)[1]}; }
+    template <bool NT = false>
+    static __device__ __forceinline__ raw load_raw(const void *p) {
+        return raw{stream_load<NT>((const v4f *)p), stream_load<NT>((const v4f *)p + 1)};
+    }
     static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {

@@ -149,7 +149,8 @@ struct ExpertTable {
 
 // a[e] = row tiles (of `bm` rows) of experts before e, b[e] = 128-row tiles of the padded token
 // axis before e, for e in [0, E]; n = E.
-__device__ __forceinline__ void build_row_tile_table(ExpertTable &tb, const int32_t *__restrict__ offsets, int E, int bm) {
+__device__ __forceinline__ void build_row_tile_table(int *__restrict__ tab_a, int *__restrict__ tab_b,
+                                                     const int32_t *__restrict__ offsets, int E, int bm) {
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
         int carry_t = 0, carry_p = 0;
@@ -159,16 +160,15 @@ __device__ __forceinline__ void build_row_tile_table(ExpertTable &tb, const int3
             const int tiles = (rows + bm - 1) / bm, pads = (rows + 127) / 128;
             const int it = wave_incl_scan(tiles, lane), ip = wave_incl_scan(pads, lane);
             if (e < E) {
-                tb.a[e] = carry_t + it - tiles;
-                tb.b[e] = carry_p + ip - pads;
+                tab_a[e] = carry_t + it - tiles;
+                tab_b[e] = carry_p + ip - pads;
             }
             carry_t += __shfl(it, 63, 64);
             carry_p += __shfl(ip, 63, 64);
         }
         if (lane == 0) {
-            tb.a[E] = carry_t;
-            tb.b[E] = carry_p;
-            tb.n = E;
+            tab_a[E] = carry_t;
+            tab_b[E] = carry_p;
         }
     }
     __syncthreads();
@@ -233,17 +233,17 @@ struct GroupedProblem {
     // the fused epilogues issue a different number of stores per lane (row and column masks): see persistent_gemm
     static constexpr bool EARLY_WAIT = MODE == MODE_GEMM1 || MODE == MODE_DGRAD2;
 
-    const ExpertTable *tb;  // row-tile prefix table in LDS, or nullptr (more experts than it holds)
+    const int *tab_a, *tab_b;  // row-tile prefix tables in LDS (build_row_tile_table), or nullptr (more experts than they hold)
 
-    __device__ GroupedProblem(const GroupedArgs &a, const ExpertTable *table)
-        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0), scan_pad(0), tb(table) {}
+    __device__ GroupedProblem(const GroupedArgs &a, const int *table_a, const int *table_b)
+        : p(a), next_id(blockIdx.x), kb_end(a.K >> 5), scan_e(0), scan_tiles(0), scan_pad(0), tab_a(table_a), tab_b(table_b) {}
 
     __device__ __forceinline__ bool next(Tile &t) {
         // With the table the number of real row tiles is known: ids cover exactly those, so the
         // contiguous id ranges of the XCDs hold equal shares of real work.  (Over the host's bound,
         // rows / BM + E row tiles, the ranges of the last XCDs hold only ids past the end: with 64
         // experts at the benchmark's routing one XCD of eight had nothing to do.)
-        const int total = p.tiles_n * (tb ? tb->a[p.E] : p.tbound);
+        const int total = p.tiles_n * (tab_a ? tab_a[p.E] : p.tbound);
         const int per_xcd = total >> 3;
         while (next_id < total) {
             int id = next_id;
@@ -253,18 +253,18 @@ struct GroupedProblem {
             if (id < (per_xcd << 3)) id = (id & 7) * per_xcd + (id >> 3);
             const int rt = id / p.tiles_n;
             const int tn = id - rt * p.tiles_n;
-            if (tb) {
+            if (tab_a) {
                 int lo = 0, hi = p.E;  // a[lo] <= rt < a[hi]: the last expert that starts at or before rt owns it
                 while (hi - lo > 1) {
                     const int mid = (lo + hi) >> 1;
-                    if (tb->a[mid] <= rt) lo = mid;
+                    if (tab_a[mid] <= rt) lo = mid;
                     else hi = mid;
                 }
-                const int first = tb->a[lo];
+                const int first = tab_a[lo];
                 t.expert = lo;
                 t.row0 = p.offsets[lo] + (rt - first) * S::BM;
                 t.end = p.offsets[lo + 1];
-                t.ppos = tb->b[lo] * 128 + (rt - first) * S::BM;
+                t.ppos = tab_b[lo] * 128 + (rt - first) * S::BM;
                 t.n0 = tn * N_PER_TILE;
                 t.kt0 = 0;
                 t.kt1 = p.K >> 7;
@@ -392,6 +392,8 @@ struct GroupedProblem {
     __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT],
                                                   const LdsScratch &lds) const {
         static_assert(S::MT % 2 == 0 && N_PER_TILE * S::BM <= S::DATA_A, "token-axis staging: one A half holds the tile");
+        static_assert(S::NT == 8 && S::BM % 128 == 0, "four gate and four value sub-tiles per lane; whole 128-token tiles");
+        constexpr int CH = S::BM / 16;  // 16-byte chunks of a staged column (its BM tokens)
         const int hblock = t.n0 + L.wn * (S::WTN / 2) + 32 * (L.r16 >> 3);  // the 32 hidden units of 8 lanes
         const int h = t.n0 + L.wn * (S::WTN / 2) + 4 * L.r16;
         const bool tok = p.htq != nullptr;
@@ -455,35 +457,37 @@ struct GroupedProblem {
                 for (int ii = 0; ii < 2; ii++) {
                     const int row = L.wm * S::WTM + 16 * (2 * blk + ii) + 4 * L.g;  // 4 consecutive rows: one dword
                     const uint32_t w = pack4_e4m3(a[ii][0][e] * inv, a[ii][1][e] * inv, a[ii][2][e] * inv, a[ii][3][e] * inv);
-                    // column-major, 256 bytes per hidden unit, 16-byte chunks XOR-swizzled by the lane's r16
-                    *(uint32_t *)(lds.a + col * S::BM + ((((row >> 4) ^ (col >> 2)) & 15) << 4) + (row & 15)) = w;
+                    // column-major, BM bytes per hidden unit, 16-byte chunks XOR-swizzled by the lane's r16
+                    *(uint32_t *)(lds.a + col * S::BM + ((((row >> 4) ^ (col >> 2)) & (CH - 1)) << 4) + (row & 15)) = w;
                 }
                 if (L.g == 0) lds.b[col * (S::BM / 32) + L.wm * (S::WTM / 32) + blk] = (uint8_t)byte;
             }
         }
         if (!tok) return -1;
         __syncthreads();
-        // 16 consecutive lanes write the 256 bytes of one hidden unit's 256 tokens; a 128-row half
+        // CH consecutive lanes write the BM bytes of one hidden unit's BM tokens; a 128-row part
         // that starts past the expert's rows belongs to the next expert's padding and is skipped
         // wave-uniform and lane-dependent parts of the addresses below are rebuilt here (scalar register,
         // opaque lane id): as invariants of the tile loop they were spilled and reloaded behind full waits
         const int64_t pbase = __builtin_amdgcn_readfirstlane(t.ppos);
         const int o_tid = opaque(L).tid;
+        static_assert((N_PER_TILE * S::BM / 16) % S::NTHR == 0, "whole rounds of 16-byte chunks");
 #pragma unroll
         for (int k = 0; k < N_PER_TILE * S::BM / 16 / S::NTHR; k++) {
             const int q = o_tid + k * S::NTHR;
-            const int col = q >> 4, ch = q & 15;
-            const bool half_ok = t.row0 + (ch >> 3) * 128 < t.end;
-            if (t.n0 + col < p.N && half_ok) {
-                const v4i w = *(const v4i *)(lds.a + col * S::BM + (((ch ^ (col >> 2)) & 15) << 4));
+            const int col = q / CH, ch = q % CH;
+            const bool part_ok = t.row0 + (ch >> 3) * 128 < t.end;
+            if (t.n0 + col < p.N && part_ok) {
+                const v4i w = *(const v4i *)(lds.a + col * S::BM + (((ch ^ (col >> 2)) & (CH - 1)) << 4));
                 *(v4i *)(p.htq + (int64_t)(t.n0 + col) * p.ldhtq + pbase + ch * 16) = w;
             }
         }
         if (o_tid < N_PER_TILE && t.n0 + o_tid < p.N) {
             const uint32_t *src = (const uint32_t *)(lds.b + o_tid * (S::BM / 32));
             uint8_t *dst = p.hts + (int64_t)(t.n0 + o_tid) * p.ldhts + (pbase >> 5);
-            *(uint32_t *)dst = src[0];
-            if (t.row0 + 128 < t.end) *(uint32_t *)(dst + 4) = src[1];
+#pragma unroll
+            for (int part = 0; part < S::BM / 128; part++)  // a dword of scale bytes per 128 tokens
+                if (t.row0 + part * 128 < t.end) *(uint32_t *)(dst + 4 * part) = src[part];
         }
         return -1;
     }
@@ -526,7 +530,9 @@ struct GroupedProblem {
                                                    const LdsScratch &lds) const {
         static_assert(S::MT % 2 == 0 && (S::BN / 2) * S::BM <= S::DATA_A && (S::BN / 2) * S::BM <= S::DATA_B &&
                           2 * (S::BN / 2) * (S::BM / 32) <= 4 * S::PA * 4,
-                      "token-axis staging: 128 columns per pass, two passes in flight");
+                      "token-axis staging: half the tile's columns per pass, two passes in flight");
+        static_assert(S::NT == 8 && S::BM % 128 == 0, "eight consecutive columns per lane; whole 128-token tiles");
+        constexpr int CH = S::BM / 16;  // 16-byte chunks of a staged column (its BM tokens)
         const bool tok = p.htq != nullptr;
         uint32_t keep[2][S::MT][4][4];  // [gate | value][slab][row][pair of columns]
         const int H = p.N;
@@ -689,23 +695,24 @@ struct GroupedProblem {
                     for (int ii = 0; ii < 2; ii++) {
                         const int row = L.wm * S::WTM + 16 * (2 * blk + ii) + 4 * o_g;  // 4 consecutive rows: one dword
                         const uint32_t w = pack4_e4m3(val[ii][0] * inv, val[ii][1] * inv, val[ii][2] * inv, val[ii][3] * inv);
-                        // column-major, 256 bytes per column, 16-byte chunks XOR-swizzled by the lane's r16
-                        *(uint32_t *)(codes + col * S::BM + ((((row >> 4) ^ (col >> 2)) & 15) << 4) + (row & 15)) = w;
+                        // column-major, BM bytes per column, 16-byte chunks XOR-swizzled by the lane's r16
+                        *(uint32_t *)(codes + col * S::BM + ((((row >> 4) ^ (col >> 2)) & (CH - 1)) << 4) + (row & 15)) = w;
                     }
                     if (o_g == 0) bytes[col * (S::BM / 32) + L.wm * (S::WTM / 32) + blk] = (uint8_t)byte;
                 }
             }
             __syncthreads();
-            // 16 consecutive lanes write the 256 bytes of one column's 256 tokens; a 128-row half
+            // CH consecutive lanes write the BM bytes of one column's BM tokens; a 128-row part
             // that starts past the expert's rows belongs to the next expert's padding and is skipped
+            static_assert(((S::BN / 2) * S::BM / 16) % S::NTHR == 0, "whole rounds of 16-byte chunks");
 #pragma unroll
             for (int k = 0; k < (S::BN / 2) * S::BM / 16 / S::NTHR; k++) {
                 const int q = o_tid + k * S::NTHR;
-                const int col = q >> 4, ch = q & 15;
+                const int col = q / CH, ch = q % CH;
                 const int hcol = t.n0 + 8 * (col >> 2) + 4 * sub + (col & 3);
-                const bool half_ok = t.row0 + (ch >> 3) * 128 < t.end;
-                if (hcol < H && half_ok) {
-                    const v4i w = *(const v4i *)(codes + col * S::BM + (((ch ^ (col >> 2)) & 15) << 4));
+                const bool part_ok = t.row0 + (ch >> 3) * 128 < t.end;
+                if (hcol < H && part_ok) {
+                    const v4i w = *(const v4i *)(codes + col * S::BM + (((ch ^ (col >> 2)) & (CH - 1)) << 4));
                     *(v4i *)(p.htq + (int64_t)(half * H + hcol) * p.ldhtq + pbase + ch * 16) = w;
                 }
             }
@@ -714,8 +721,9 @@ struct GroupedProblem {
                 if (hcol < H) {
                     const uint32_t *src = (const uint32_t *)(bytes + o_tid * (S::BM / 32));
                     uint8_t *dst = p.hts + (int64_t)(half * H + hcol) * p.ldhts + (pbase >> 5);
-                    *(uint32_t *)dst = src[0];
-                    if (t.row0 + 128 < t.end) *(uint32_t *)(dst + 4) = src[1];
+#pragma unroll
+                    for (int part = 0; part < S::BM / 128; part++)  // a dword of scale bytes per 128 tokens
+                        if (t.row0 + part * 128 < t.end) *(uint32_t *)(dst + 4 * part) = src[part];
                 }
             }
         }
@@ -774,15 +782,36 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t *__restrict
     *(v4i *)(out + t * ldo + c) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
 }
 
+// Experts the row-tile tables of a workgroup hold.  Two workgroups share a CU's 160 KB under the 128 x 128 shape: their
+// stage buffers take 2 x 73 KB, which leaves room for 512 experts each.
+template <typename S>
+constexpr int row_table_max() { return S::BM + S::BN > 256 ? MX_TABLE_MAX : 512; }
+
+template <typename S, int MODE, int CDT, int K512>
+__device__ __forceinline__ void grouped_body(const GroupedArgs &args, uint8_t *smem) {
+    constexpr int TMAX = row_table_max<S>();
+    __shared__ int table_a[TMAX + 1], table_b[TMAX + 1];
+    const bool tabled = args.E <= TMAX;
+    if (tabled) build_row_tile_table(table_a, table_b, args.offsets, args.E, S::BM);
+    GroupedProblem<S, MODE, CDT> prob(args, tabled ? table_a : nullptr, tabled ? table_b : nullptr);
+    persistent_gemm<S, K512>(prob, smem);
+}
+
 template <typename S, int MODE, int CDT, int K512>
 __global__ __launch_bounds__(S::NTHR) void grouped_kernel(GroupedArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    __shared__ ExpertTable table;
-    const bool tabled = args.E <= MX_TABLE_MAX;
-    if (tabled) build_row_tile_table(table, args.offsets, args.E, S::BM);
-    GroupedProblem<S, MODE, CDT> prob(args, tabled ? &table : nullptr);
-    persistent_gemm<S, K512>(prob, smem);
+    grouped_body<S, MODE, CDT, K512>(args, smem);
 }
+
+#ifdef MX_BENCH_VARIANTS
+// The same body on the 128 x 128 tile of four waves (one per SIMD), two workgroups resident per CU, so that one
+// workgroup's epilogue can run while the other one's MFMAs do.  The register budget is the one of two waves per SIMD.
+template <typename S, int MODE, int CDT, int K512>
+__global__ __launch_bounds__(S::NTHR) __attribute__((amdgpu_waves_per_eu(2, 2))) void grouped_pair_kernel(GroupedArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    grouped_body<S, MODE, CDT, K512>(args, smem);
+}
+#endif
 
 // Slow path for shapes the tiled kernel does not take (PLAIN only): one thread per output element.
 template <int CDT>
@@ -1166,22 +1195,51 @@ static bool tiled_ok(const GroupedArgs &a, int64_t a_rows) {
            a.stride_wse % 4 == 0 && a_rows * a.ldx < ((int64_t)1 << 32) && (int64_t)a.N * 2 * a.ldw < ((int64_t)1 << 32);
 }
 
-template <int MODE, int CDT>
-static int launch_grouped(GroupedArgs a, hipStream_t st) {
-    typedef Big S;
+// 128 x 128 x 128 tile, 4 waves as 4 (M) x 1 (N), one per SIMD: a wave owns 32 x 128 -- the same eight consecutive N per
+// lane as under Big, so the fused epilogues' column logic is shared -- and two workgroups fit a CU (2 x 73 KB of LDS,
+// 256 registers per lane each).  Twice the operand bytes per flop of Big: for the fused expert epilogues only, whose
+// vector ALU work dwarfs their short K loops.
+typedef GemmShape<128, 128, 4, 1> Slim;
+
+// Built into the variants library only (-DMX_BENCH_VARIANTS), where it replaces Big for the two fused expert kernels:
+// bit-identical outputs, measured slower at the benchmark's routing (GEMM1 148 -> 185 us, GEMM2-dgrad 192 -> 209 us).
+// The eight waves of a CU issue the same vector ALU work either way, and the K loops of a 128 x 128 tile, whose copies
+// must land within a stage of 512 MFMA clocks, cost more than their overlap with the other workgroup's epilogue returns.
+#ifdef MX_BENCH_VARIANTS
+#define MX_EXPERT_SLIM 1
+#else
+#define MX_EXPERT_SLIM 0
+#endif
+
+template <typename S, int MODE, int CDT>
+static int launch_grouped_shape(GroupedArgs a, hipStream_t st) {
     constexpr int npt = MODE == MODE_GEMM1 ? S::BN / 2 : S::BN;
+    constexpr bool pair = S::NW == 4;  // two workgroups per CU
     a.tiles_n = (a.N + npt - 1) / npt;
     a.tbound = (a.M + S::BM - 1) / S::BM + a.E;
     const int64_t work = (int64_t)a.tiles_n * a.tbound;
     if (work >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
     const bool k512 = a.K % 512 == 0 && aligned(a.xs, 16) && aligned(a.ws, 16) && a.ldxs % 16 == 0 &&
                       a.ldws % 16 == 0 && a.stride_wse % 16 == 0;
-    const int cus = num_cus();
-    dim3 grid((unsigned)(work < cus ? work : cus)), block(S::NTHR);
-    const int rc = k512 ? launch_with_lds<grouped_kernel<S, MODE, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
-                        : launch_with_lds<grouped_kernel<S, MODE, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
+    const int wgs = num_cus() * (pair ? 2 : 1);
+    dim3 grid((unsigned)(work < wgs ? work : wgs)), block(S::NTHR);
+    int rc;
+#ifdef MX_BENCH_VARIANTS
+    if constexpr (pair)
+        rc = k512 ? launch_with_lds<grouped_pair_kernel<S, MODE, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+                  : launch_with_lds<grouped_pair_kernel<S, MODE, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
+    else
+#endif
+        rc = k512 ? launch_with_lds<grouped_kernel<S, MODE, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+                  : launch_with_lds<grouped_kernel<S, MODE, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
     if (rc != MX_OK) return rc;
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+template <int MODE, int CDT>
+static int launch_grouped(const GroupedArgs &a, hipStream_t st) {
+    if constexpr (MX_EXPERT_SLIM && (MODE == MODE_GEMM1 || MODE == MODE_DGRAD2)) return launch_grouped_shape<Slim, MODE, CDT>(a, st);
+    else return launch_grouped_shape<Big, MODE, CDT>(a, st);
 }
 
 template <int MODE>

@@ -10,47 +10,65 @@ namespace mx {
 
 int num_cus();  // mx_gemm.hip
 
-// 16 bytes per lane per load, UNROLL loads in flight per lane, grid-stride over whole chunks.
+// 16 bytes per lane per access, UNROLL accesses of every stream in flight per lane, grid-stride over whole chunks.
+// What is swept (mx_ubench_stream_cfg): threads per workgroup, UNROLL, workgroups per CU (0: one chunk per workgroup,
+// no loop) and whether loads / stores carry the non-temporal hint.  The default entry point runs one fixed point.
 constexpr int STREAM_THREADS = 256;
 constexpr int STREAM_UNROLL = 4;
+constexpr int STREAM_MAX_THREADS = 1024;
 
-__device__ __forceinline__ v4i nt_load(const v4i *p) { return __builtin_nontemporal_load(p); }
-__device__ __forceinline__ void nt_store(v4i *p, v4i v) { __builtin_nontemporal_store(v, p); }
+template <bool NT>
+__device__ __forceinline__ v4i ld16(const v4i *p) { return NT ? __builtin_nontemporal_load(p) : *p; }
+template <bool NT>
+__device__ __forceinline__ void st16(v4i *p, v4i v) {
+    if (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
 
 // kind 0: read only (a); every thread folds what it read into one dword of `c` (one per thread)
-// kind 1: copy c = a
-// kind 2: triad c = a + 2 b on fp32
+// kind 1: copy c = a                                                            (1 : 1)
+// kind 2: triad c = a + 2 b on fp32                                             (2 : 1, with arithmetic)
 // kind 3: 2 : 1 mix -- reads two 16-byte vectors (a[2i], a[2i+1]) and writes one (their byte-wise fold) to c[i]:
-//         the traffic of a 16-bit -> 8-bit cast without its arithmetic
-template <int KIND>
-__global__ __launch_bounds__(STREAM_THREADS) void stream_kernel(const v4i *__restrict__ a, const v4i *__restrict__ b,
-                                                                v4i *__restrict__ c, int64_t n_out) {
-    const int64_t stride = (int64_t)gridDim.x * STREAM_THREADS;
-    int64_t i = (int64_t)blockIdx.x * STREAM_THREADS + threadIdx.x;
+//         the traffic of a 16-bit -> 8-bit cast without its arithmetic, one input stream
+// kind 4: 2 : 1 mix from two input streams -- c[i] = fold(a[i], a[n + i]) (a holds 2 n vectors)
+// kind 5: 3 : 2 mix -- reads a[i], a[n + i], a[2 n + i], writes c[i] and c[n + i] (a holds 3 n vectors, c 2 n):
+//         the traffic of the SwiGLU' quantizer (three 16-bit inputs, four 8-bit outputs)
+template <int KIND, int UNROLL, bool NTL, bool NTS>
+__global__ __launch_bounds__(STREAM_MAX_THREADS) void stream_kernel(const v4i *__restrict__ a, const v4i *__restrict__ b,
+                                                                    v4i *__restrict__ c, int64_t n_out) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     v4i fold = {0, 0, 0, 0};
-    for (; i + (STREAM_UNROLL - 1) * stride < n_out; i += STREAM_UNROLL * stride) {
-        v4i x[STREAM_UNROLL], y[STREAM_UNROLL];
+    for (; i + (UNROLL - 1) * stride < n_out; i += UNROLL * stride) {
+        v4i x[UNROLL], y[UNROLL], z[UNROLL];
 #pragma unroll
-        for (int u = 0; u < STREAM_UNROLL; u++) {
+        for (int u = 0; u < UNROLL; u++) {
+            const int64_t at = i + u * stride;
             if (KIND == 3) {
-                x[u] = nt_load(a + 2 * (i + u * stride));
-                y[u] = nt_load(a + 2 * (i + u * stride) + 1);
+                x[u] = ld16<NTL>(a + 2 * at);
+                y[u] = ld16<NTL>(a + 2 * at + 1);
             } else {
-                x[u] = nt_load(a + i + u * stride);
-                if (KIND == 2) y[u] = nt_load(b + i + u * stride);
+                x[u] = ld16<NTL>(a + at);
+                if (KIND == 2) y[u] = ld16<NTL>(b + at);
+                if (KIND >= 4) y[u] = ld16<NTL>(a + n_out + at);
+                if (KIND == 5) z[u] = ld16<NTL>(a + 2 * n_out + at);
             }
         }
 #pragma unroll
-        for (int u = 0; u < STREAM_UNROLL; u++) {
+        for (int u = 0; u < UNROLL; u++) {
+            const int64_t at = i + u * stride;
             if (KIND == 0) {
                 fold ^= x[u];
             } else if (KIND == 1) {
-                nt_store(c + i + u * stride, x[u]);
+                st16<NTS>(c + at, x[u]);
             } else if (KIND == 2) {
                 v4f fa = __builtin_bit_cast(v4f, x[u]), fb = __builtin_bit_cast(v4f, y[u]);
-                nt_store(c + i + u * stride, __builtin_bit_cast(v4i, fa + 2.0f * fb));
+                st16<NTS>(c + at, __builtin_bit_cast(v4i, fa + 2.0f * fb));
+            } else if (KIND == 5) {
+                st16<NTS>(c + at, (x[u] & 0x00FF00FF) | ((y[u] & 0x00FF00FF) << 8));
+                st16<NTS>(c + n_out + at, (z[u] & 0x00FF00FF) | ((y[u] & 0xFF00FF00)));
             } else {
-                nt_store(c + i + u * stride, (x[u] & 0x00FF00FF) | ((y[u] & 0x00FF00FF) << 8));
+                st16<NTS>(c + at, (x[u] & 0x00FF00FF) | ((y[u] & 0x00FF00FF) << 8));
             }
         }
     }
@@ -58,9 +76,36 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_kernel(const v4i *__res
         if (KIND == 0) fold ^= a[i];
         else if (KIND == 1) c[i] = a[i];
         else if (KIND == 2) c[i] = __builtin_bit_cast(v4i, __builtin_bit_cast(v4f, a[i]) + 2.0f * __builtin_bit_cast(v4f, b[i]));
-        else c[i] = (a[2 * i] & 0x00FF00FF) | ((a[2 * i + 1] & 0x00FF00FF) << 8);
+        else if (KIND == 3) c[i] = (a[2 * i] & 0x00FF00FF) | ((a[2 * i + 1] & 0x00FF00FF) << 8);
+        else if (KIND == 4) c[i] = (a[i] & 0x00FF00FF) | ((a[n_out + i] & 0x00FF00FF) << 8);
+        else {
+            c[i] = (a[i] & 0x00FF00FF) | ((a[n_out + i] & 0x00FF00FF) << 8);
+            c[n_out + i] = (a[2 * n_out + i] & 0x00FF00FF) | (a[n_out + i] & 0xFF00FF00);
+        }
     }
-    if (KIND == 0) ((int *)c)[(int64_t)blockIdx.x * STREAM_THREADS + threadIdx.x] = fold[0] ^ fold[1] ^ fold[2] ^ fold[3];
+    if (KIND == 0) ((int *)c)[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = fold[0] ^ fold[1] ^ fold[2] ^ fold[3];
+}
+
+template <int KIND, int UNROLL>
+static void launch_stream(bool ntl, bool nts, dim3 grid, dim3 block, hipStream_t st, const v4i *a, const v4i *b, v4i *c,
+                          int64_t n) {
+    if (ntl && nts) stream_kernel<KIND, UNROLL, true, true><<<grid, block, 0, st>>>(a, b, c, n);
+    else if (ntl) stream_kernel<KIND, UNROLL, true, false><<<grid, block, 0, st>>>(a, b, c, n);
+    else if (nts) stream_kernel<KIND, UNROLL, false, true><<<grid, block, 0, st>>>(a, b, c, n);
+    else stream_kernel<KIND, UNROLL, false, false><<<grid, block, 0, st>>>(a, b, c, n);
+}
+
+template <int KIND>
+static int launch_stream_unroll(int unroll, bool ntl, bool nts, dim3 grid, dim3 block, hipStream_t st, const v4i *a,
+                                const v4i *b, v4i *c, int64_t n) {
+    switch (unroll) {
+    case 1: launch_stream<KIND, 1>(ntl, nts, grid, block, st, a, b, c, n); break;
+    case 2: launch_stream<KIND, 2>(ntl, nts, grid, block, st, a, b, c, n); break;
+    case 4: launch_stream<KIND, 4>(ntl, nts, grid, block, st, a, b, c, n); break;
+    case 8: launch_stream<KIND, 8>(ntl, nts, grid, block, st, a, b, c, n); break;
+    default: return MX_EINVAL;
+    }
+    return MX_OK;
 }
 
 // Register-resident block-scaled fp8 MFMA loop: ACCS independent accumulator tiles per wave, operands that never
@@ -127,23 +172,39 @@ __global__ __launch_bounds__(512) void mfma_peak_kernel(int iters, int random, f
 
 using namespace mx;
 
-extern "C" int mx_ubench_stream(int kind, const void *a, const void *b, void *c, int64_t out_bytes, void *stream) {
-    if (kind < 0 || kind > 3 || out_bytes < 0 || out_bytes % 16) return MX_EINVAL;
+extern "C" int mx_ubench_stream_cfg(int kind, int threads, int unroll, int wgs_per_cu, int nontemporal, const void *a,
+                                    const void *b, void *c, int64_t out_bytes, void *stream) {
+    if (kind < 0 || kind > 5 || out_bytes < 0 || out_bytes % 16) return MX_EINVAL;
+    if (threads < 64 || threads > STREAM_MAX_THREADS || threads % 64 || wgs_per_cu < 0 || nontemporal < 0 || nontemporal > 3)
+        return MX_EINVAL;
     if (!a || !c || (kind == 2 && !b) || ((uintptr_t)a & 15) || ((uintptr_t)b & 15) || ((uintptr_t)c & 15)) return MX_EINVAL;
     hipStream_t st = (hipStream_t)stream;
     if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     const int64_t n = out_bytes / 16;
     // enough resident waves to cover HBM latency on every CU, few enough that the grid-stride loop does the work
-    const int64_t want = (n + STREAM_THREADS * STREAM_UNROLL - 1) / (STREAM_THREADS * STREAM_UNROLL);
-    const int64_t cap = (int64_t)num_cus() * 16;
-    const dim3 grid((unsigned)(want < 1 ? 1 : want < cap ? want : cap)), block(STREAM_THREADS);
+    const int64_t want = (n + (int64_t)threads * unroll - 1) / ((int64_t)threads * unroll);
+    const int64_t cap = wgs_per_cu ? (int64_t)num_cus() * wgs_per_cu : want;
+    if ((want < cap ? want : cap) > 0x7FFFFFFF) return MX_EUNSUPPORTED;
+    const dim3 grid((unsigned)(want < 1 ? 1 : want < cap ? want : cap)), block((unsigned)threads);
+    const bool ntl = nontemporal & 1, nts = nontemporal & 2;
+    const v4i *pa = (const v4i *)a, *pb = (const v4i *)b;
+    v4i *pc = (v4i *)c;
+    int rc;
     switch (kind) {
-    case 0: stream_kernel<0><<<grid, block, 0, st>>>((const v4i *)a, nullptr, (v4i *)c, n); break;
-    case 1: stream_kernel<1><<<grid, block, 0, st>>>((const v4i *)a, nullptr, (v4i *)c, n); break;
-    case 2: stream_kernel<2><<<grid, block, 0, st>>>((const v4i *)a, (const v4i *)b, (v4i *)c, n); break;
-    default: stream_kernel<3><<<grid, block, 0, st>>>((const v4i *)a, nullptr, (v4i *)c, n); break;
+    case 0: rc = launch_stream_unroll<0>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
+    case 1: rc = launch_stream_unroll<1>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
+    case 2: rc = launch_stream_unroll<2>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
+    case 3: rc = launch_stream_unroll<3>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
+    case 4: rc = launch_stream_unroll<4>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
+    default: rc = launch_stream_unroll<5>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
     }
+    if (rc != MX_OK) return rc;
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+extern "C" int mx_ubench_stream(int kind, const void *a, const void *b, void *c, int64_t out_bytes, void *stream) {
+    if (kind > 3) return MX_EINVAL;
+    return mx_ubench_stream_cfg(kind, STREAM_THREADS, STREAM_UNROLL, 16, 3, a, b, c, out_bytes, stream);
 }
 
 extern "C" int64_t mx_ubench_mfma(int wide, int iters, int random, float *out, int64_t out_floats, void *stream) {

@@ -303,6 +303,53 @@ def _expert_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
     return dict(out=out, pre=pre, hq=hq, hs=hs, dx=dx, dgate=dgate, dw_in=dw_in, dw_out=dw_out)
 
 
+def _unfused_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
+    """The unfused path's own arithmetic (src/kohakuwullm/kernels/mxfp8/moe_unfused.py:25-158) restated with oracle
+    primitives.  Its casts sit elsewhere than the fused graph's: `pre`, `h`, the combine's rows, `dh` and `dpre` all make
+    a 16-bit round trip between launches, SwiGLU and its derivative are PyTorch's 16-bit elementwise operators (taken
+    here from PyTorch on the CPU, autograd included), and the gate is applied to the upstream rows BEFORE the dgrad
+    quantizer (the combine's backward), not to the accumulator behind it.  WGRAD is this build's: MXFP8 on token-axis
+    blocks inside each expert's segment."""
+    e, two_h, dim = w_in.shape
+    off = offsets.tolist()
+    m = off[-1]
+    t_idx, p_idx = token_of.long()[:m], order.long()[:m]
+
+    def stacked(w):
+        q, s = ora.quantize_rows(w.reshape(-1, w.shape[-1]))
+        return q.view(*w.shape), s.view(*w.shape[:-1], w.shape[-1] // 32)
+
+    in_f, out_f = stacked(w_in), stacked(w_out)
+    in_d, out_d = stacked(w_in.transpose(1, 2).contiguous()), stacked(w_out.transpose(1, 2).contiguous())
+    act = x.dtype
+    pre = ora.grouped_gemm_nt(*ora.quantize_rows(x), *in_f, offsets, t_idx).to(act).requires_grad_(True)
+    gate_h, value = pre.chunk(2, dim=-1)
+    h = torch.nn.functional.silu(gate_h) * value  # 16-bit operators: silu rounds, the product rounds again
+    y = ora.grouped_gemm_nt(*ora.quantize_rows(h.detach()), *out_f, offsets).to(act)
+    out = ora.combine_routed(y, gate, order[:m], token_of[:m], x.shape[0])
+    # backward: combine, second product, SwiGLU (autograd of the 16-bit operators), first product
+    grad_rows, dgate = ora.combine_routed_grads(dout, y, gate, order[:m], token_of[:m])
+    dh = ora.grouped_gemm_nt(*ora.quantize_rows(grad_rows), *out_d, offsets).to(act)
+    (dpre,) = torch.autograd.grad(h, pre, dh)
+    dx_sorted = ora.grouped_gemm_nt(*ora.quantize_rows(dpre), *in_d, offsets).to(act)
+    dx = torch.zeros(x.shape[0], dim, dtype=torch.float64).index_add_(0, t_idx, dx_sorted.double())
+    dw_out = torch.zeros(e, dim, two_h // 2, dtype=torch.float64)
+    dw_in = torch.zeros(e, two_h, dim, dtype=torch.float64)
+    xg, h16 = x.float()[t_idx], h.detach().float()
+    for i in range(e):
+        lo, hi = off[i], off[i + 1]
+        if hi == lo:
+            continue
+        pad = -(hi - lo) % 32
+
+        def qc(rows):
+            return ora.quantize_cols(torch.nn.functional.pad(rows, (0, 0, 0, pad)))
+
+        dw_out[i] = ora.gemm_nt(*qc(grad_rows.float()[lo:hi]), *qc(h16[lo:hi]))
+        dw_in[i] = ora.gemm_nt(*qc(dpre.float()[lo:hi]), *qc(xg[lo:hi]))
+    return dict(out=out, dx=dx, dgate=dgate, dw_in=dw_in, dw_out=dw_out)
+
+
 @pytest.mark.parametrize("counts,top_k", [([300, 0, 1, 257, 0, 130], 2), ([256, 256], 1),
                                           ([0] * 70 + [200] + [0] * 130 + [129, 1] + [0] * 50, 1)])
 @pytest.mark.parametrize("dout_scale", [1.0, 2.0**-20])
@@ -354,14 +401,85 @@ def test_fused_experts_fwd_bwd(oracle, counts, top_k, dout_scale):
     assert oracle.rel_error(dgate, gf.grad) < 0.12
 
     # the unfused twin computes the same function through differently placed casts (16-bit h and
-    # dh round trips, the gate applied before the dgrad quantizer): its forward sits within the
-    # 16-bit round trip of the fused oracle, its gradients within the e4m3 error of the exact ones
+    # dh round trips, the gate applied before the dgrad quantizer): held to an oracle chain of ITS cast
+    # placement at the same 1e-2 as the fused graph, forward and every gradient
     out_u, dx_u, dw_in_u, dw_out_u, dgate_u = run(mxfp8_moe_experts_unfused)
-    assert oracle.rel_error(out_u, ref["out"]) < 2e-2
-    assert oracle.rel_error(dx_u, xf.grad) < 0.12
-    assert oracle.rel_error(dw_in_u, wif.grad) < 0.12
-    assert oracle.rel_error(dw_out_u, wof.grad) < 0.12
-    assert oracle.rel_error(dgate_u, gf.grad) < 0.12
+    ref_u = _unfused_oracle(oracle, x, w_in, w_out, gate, token_of, order, offsets, dout)
+    assert oracle.rel_error(out_u, ref_u["out"].double()) < TOL
+    assert oracle.rel_error(dx_u, ref_u["dx"]) < TOL
+    assert oracle.rel_error(dgate_u, ref_u["dgate"]) < TOL
+    assert oracle.rel_error(dw_out_u, ref_u["dw_out"]) < TOL
+    assert oracle.rel_error(dw_in_u, ref_u["dw_in"]) < TOL
+    assert oracle.rel_error(out_u, ref["out"]) < 2e-2  # and within the 16-bit round trips of the fused oracle
+
+
+@pytest.mark.parametrize("counts,top_k", [([300, 0, 1, 257, 0, 130], 2), ([0, 511], 1)])
+def test_fused_experts_scatter_route(oracle, counts, top_k):
+    """The atomic route of GEMM2 and GEMM1-dgrad (the reference's own: tl.atomic_add epilogues, experts.py:138-222,
+    experts_bwd.py:167-247).  The fused graph takes it when `order` is not known to be the pair index token * top_k +
+    slot -- here: a gate vector one element longer than tokens * top_k, whose last element no pair uses -- and the
+    scatter GEMM is also called on its own, with 16-bit and fp32 outputs, with and without a gate and a row index.
+    Sums of atomics: compared by norm, never bitwise."""
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, launch_scatter_gemm, mxfp8_moe_experts
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator().manual_seed(SEED + 3)
+    e, tokens, dim, hid = len(counts), 512, 256, 128
+    offsets, order, token_of = _routing(counts, top_k, tokens)
+    x = torch.randn(tokens, dim, generator=g).bfloat16()
+    w_in = (torch.randn(e, 2 * hid, dim, generator=g) * 0.06).bfloat16()
+    w_out = (torch.randn(e, dim, hid, generator=g) * 0.06).bfloat16()
+    gate = (torch.rand(tokens * top_k + 1, generator=g) * 0.5 + 0.5).bfloat16()
+    dout = torch.randn(tokens, dim, generator=g).bfloat16()
+    ref = _expert_oracle(oracle, x, w_in, w_out, gate, token_of, order, offsets, dout)
+
+    xd, wi, wo, gd = (t.to(DEV).requires_grad_(True) for t in (x, w_in, w_out, gate))
+    packed = MXFP8ExpertWeights(wi.detach(), wo.detach())
+    from kohakuwullm_amd import _lib
+
+    _lib.TIMER = []  # records the entry points the call goes through
+    try:
+        out = mxfp8_moe_experts(xd, wi, wo, gd, token_of.to(DEV), order.to(DEV), offsets.to(DEV), packed)
+        out.backward(dout.to(DEV))
+        torch.cuda.synchronize()
+        called = [name for name, *_ in _lib.TIMER]
+    finally:
+        _lib.TIMER = None
+    assert called.count("mx_experts_scatter_gemm") == 2 and "mx_experts_combine" not in called
+    assert oracle.rel_error(out.detach().cpu(), ref["out"]) < TOL
+    assert oracle.rel_error(xd.grad.cpu(), ref["dx"]) < TOL
+    assert oracle.rel_error(gd.grad.cpu(), ref["dgate"]) < TOL and gd.grad[-1] == 0
+    assert oracle.rel_error(wi.grad.cpu(), ref["dw_in"]) < TOL and oracle.rel_error(wo.grad.cpu(), ref["dw_out"]) < TOL
+
+    # the entry point on its own: out[token_of[m]] += scale(m) * (a[index[m] or m] . w[e(m)]^T)
+    m = sum(counts)
+    hq, hs = ref["hq"], ref["hs"]  # the oracle's h codes: sorted rows, K = hid
+    wq, ws = oracle.quantize_rows(w_out.reshape(-1, hid))
+    wq, ws = wq.view(e, dim, hid), ws.view(e, dim, hid // 32)
+    y = oracle.grouped_gemm_nt(hq, hs, wq, ws, offsets)  # (m, dim) fp64
+    t_idx, p_idx = token_of.long()[:m], order.long()[:m]
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    # (16-bit outputs only: the adds are packed 16-bit atomics; the gate in the output's type or in fp32)
+    for out_dtype, gate_dtype in ((torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32), (torch.float16, None)):
+        gate_t = gate.to(gate_dtype) if gate_dtype else None
+        scale = gate_t.double()[p_idx] if gate_dtype else torch.ones(m, dtype=torch.float64)
+        want = torch.zeros(tokens, dim, dtype=torch.float64).index_add_(0, t_idx, y * scale[:, None])
+        got = torch.zeros(tokens, dim, device=DEV, dtype=out_dtype)
+        launch_scatter_gemm(*_dev(hq, hs), *_dev(wq, ws), got, dev(token_of), dev(order) if gate_dtype else None,
+                            dev(gate_t) if gate_dtype else None, dev(offsets))
+        assert oracle.rel_error(got.cpu(), want) < TOL, (out_dtype, gate_dtype)
+    with pytest.raises(ValueError):  # an fp32 output is refused, not mis-added
+        launch_scatter_gemm(*_dev(hq, hs), *_dev(wq, ws), torch.zeros(tokens, dim, device=DEV), dev(token_of), None, None,
+                            dev(offsets))
+    # with a row index: a[index[m]] in place of a[m] (the quantized token rows gathered inside the kernel)
+    xq, xs = oracle.quantize_rows(x)
+    wq1, ws1 = oracle.quantize_rows(w_in.reshape(-1, dim))
+    wq1, ws1 = wq1.view(e, 2 * hid, dim), ws1.view(e, 2 * hid, dim // 32)
+    want = torch.zeros(tokens, 2 * hid, dtype=torch.float64).index_add_(
+        0, t_idx, oracle.grouped_gemm_nt(xq, xs, wq1, ws1, offsets, t_idx))
+    got = torch.zeros(tokens, 2 * hid, device=DEV, dtype=torch.bfloat16)
+    launch_scatter_gemm(*_dev(xq, xs), *_dev(wq1, ws1), got, dev(token_of), None, None, dev(offsets), index=dev(token_of))
+    assert oracle.rel_error(got.cpu(), want) < TOL
 
 
 def test_gemm1_intermediates(oracle):
@@ -466,6 +584,49 @@ def test_gemm2_dgrad_token_axis(oracle):
         assert not ptq1.view(torch.uint8).cpu()[:, ~valid].any()  # nothing is written past the experts' tiles
         with pytest.raises(Exception):
             run(False, False)  # neither output asked for
+
+
+@pytest.mark.parametrize("counts,hid", [([200, 0, 56, 300], 160), ([1, 700], 544), ([130] * 5, 256)])
+def test_expert_kernels_on_small_tiles_agree(counts, hid):
+    """The variants library runs the two fused expert kernels on 128 x 128 tiles, two workgroups per CU: every element
+    contracts the same K sequence and goes through the same epilogue arithmetic, so every output of GEMM1 and of
+    GEMM2-dgrad equals the shipped kernels' bit for bit (dgate, a sum of atomics, by norm)."""
+    from kohakuwullm_amd import _lib
+    from kohakuwullm_amd.kernels.mxfp8.grouped import padded_rows
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, launch_gemm1, launch_gemm2_dgrad
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator().manual_seed(SEED + 11)
+    e, dim, top_k = len(counts), 256, 1
+    tokens = sum(counts) + 40
+    offsets, order, token_of = (t.to(DEV) for t in _routing(counts, top_k, tokens))
+    m = sum(counts)
+    mpad = padded_rows(m, e)
+    x = torch.randn(tokens, dim, generator=g).bfloat16().to(DEV)
+    dout = torch.randn(tokens, dim, generator=g).bfloat16().to(DEV)
+    gate = (torch.rand(tokens, generator=g) * 0.5 + 0.5).bfloat16().to(DEV)
+    packed = MXFP8ExpertWeights((torch.randn(e, 2 * hid, dim, generator=g) * 0.06).bfloat16().to(DEV),
+                                (torch.randn(e, dim, hid, generator=g) * 0.06).bfloat16().to(DEV))
+    xq, xs = quantize_mx(x)
+    dq, ds = quantize_mx(dout)
+
+    def run():
+        z = lambda *shape, dtype=torch.uint8: torch.zeros(*shape, device=DEV, dtype=dtype)  # noqa: E731
+        hq, hs, pre = z(m, hid, dtype=F8), z(m, hid // 32), z(m, 2 * hid, dtype=torch.bfloat16)
+        htq, hts = z(hid, mpad, dtype=F8), z(hid, mpad // 32)
+        launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hid, dim, torch.bfloat16, htq, hts)
+        dpre, dpq, dps = z(m, 2 * hid, dtype=torch.bfloat16), z(m, 2 * hid, dtype=F8), z(m, 2 * hid // 32)
+        ptq, pts, dgate = z(2 * hid, mpad, dtype=F8), z(2 * hid, mpad // 32), z(tokens, dtype=torch.float32)
+        launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets, ptq, pts)
+        torch.cuda.synchronize()
+        return [t.view(torch.uint8) if t.dtype == F8 else t for t in (hq, hs, pre, htq, hts, dpre, dpq, dps, ptq, pts)], dgate
+
+    shipped, dgate = run()
+    with _lib.variants_library():
+        small, dgate_small = run()
+    for name, a, b in zip("hq hs pre htq hts dpre dpq dps ptq pts".split(), shipped, small):
+        assert torch.equal(a, b), name
+    assert float((dgate - dgate_small).norm() / dgate.norm()) < 1e-5
 
 
 def test_expert_call_contract():
@@ -576,11 +737,15 @@ def test_moe_module_reference_defaults(oracle):
     route_on = torch.randn(200, 256, device=DEV)
     with torch.autocast("cuda", dtype=torch.bfloat16):
         assert not torch.equal(moe(x, route_on=route_on), moe(x))
-    # fp32 activations outside autocast: the routed MXFP8 path answers in bf16, a 16-bit shared expert (fp32 weights,
-    # never swapped) in fp32, and their sum takes the promoted dtype, as in the reference's forward
+    # outside autocast the sum of the routed and the shared branch takes the promoted dtype, as in the reference's
+    # forward: fp32 activations through the 16-bit arm stay fp32; the MXFP8 arm refuses them (the compute dtype is the
+    # caller's to choose) and answers 16-bit activations of a 16-bit module in kind
     plain = MoEMLP(256, hidden=128, num_experts=16, top_k=4).to(DEV)
-    plain.enable_mxfp8()
     assert plain(x).dtype == torch.float32
+    plain.enable_mxfp8()
+    with pytest.raises(ValueError, match="compute dtype"):
+        plain(x)
+    assert plain.to(torch.bfloat16)(x.bfloat16()).dtype == torch.bfloat16
     # the per-expert loop is the eager test arm: the swap refuses it and says why
     loop = MoEMLP(256, hidden=128, num_experts=4, top_k=2, num_shared=0, dense_fallback=True).to(DEV)
     rep = swap_mxfp8(loop)
