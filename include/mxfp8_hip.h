@@ -169,7 +169,7 @@ int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, in
  * y = x * rstd * weight (fp32; weight NULL: 1).  Any of three results, from one pass over x:
  * out (M,K) in x_dtype (NULL: not written), rstd (M) fp32 for the backward (NULL: not
  * written), and (q,s) = y quantized along K from the fp32 values (both NULL: not written;
- * K % 32 == 0 when given).  At least one of out and q.  weight is x_dtype or fp32.
+ * K % 32 == 0 when given).  At least one of the three.  weight is x_dtype or fp32.
  * The sum of squares is accumulated in fp64, the rest is fp32 in the reference's order.
  * Replaces _rmsnorm_fwd with QUANT (src/kohakuwullm/kernels/elementwise/rmsnorm.py:20-84;
  * host side rms_norm_mx :239-246, rms_norm :232-236) and _rmsnorm_mx_kernel / rmsnorm_mx
@@ -179,6 +179,22 @@ int mx_swiglu_bwd_quantize_dual(const void *dh, int64_t lddh, const void *gu, in
 int mx_rmsnorm_quantize(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                         const void *weight, int w_dtype, float eps, void *out, int64_t ldo, float *rstd,
                         uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, void *stream);
+
+/*
+ * RMSNorm as a producer of BOTH MXFP8 operands of the linear layer behind it: y = x * rstd * weight in fp32 as in
+ * mx_rmsnorm_quantize, quantized along K into (q,s) (M,K), (M,K/32) -- the layer's forward operand, bit-identical to
+ * mx_rmsnorm_quantize's -- and along the tokens into (qT,sT) (K,M), (K,M/32) -- the operand of its weight gradient, the
+ * column quantizer applied to the same fp32 y.  Neither the 16-bit normalized activation nor its transpose is written.
+ * Two launches: the rows' rstd (M floats, the caller's buffer: also what mx_rmsnorm_backward takes), then 128 x 128
+ * tiles of x scaled on the way in.  M % 32 == 0, K % 32 == 0; ldqT == 128 with M > 128 selects the stage-major layout
+ * of mx_quantize_dual for qT.  weight: any of the three dtypes, or NULL.
+ * No counterpart in the reference, which emits the row-axis pair only (rmsnorm_mx,
+ * src/kohakuwullm/kernels/mxfp8/fused_act.py:104-175) and quantizes the activation a second time for WGRAD
+ * (src/kohakuwullm/kernels/mxfp8/linear.py:111).
+ */
+int mx_rmsnorm_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void *weight,
+                             int w_dtype, float eps, float *rstd, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds,
+                             uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream);
 
 /*
  * RMSNorm backward: dx = (dy - xhat * mean_k(dy * xhat)) * rstd with dy = dout * weight and

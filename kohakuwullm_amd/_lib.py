@@ -55,6 +55,8 @@ SIGNATURES = {
         _ci, [_p, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _ci, _i64, _i64, _i64, _i64, _p, _i64, _p]),
     "mx_rmsnorm_quantize": (
         _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, ctypes.c_float, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
+    "mx_rmsnorm_quantize_dual": (
+        _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, ctypes.c_float, _p, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p]),
     "mx_rmsnorm_backward": (
         _ci, [_p, _ci, _i64, _i64, _i64, _p, _ci, _p, _i64, _p, _p, _i64, _p, _i64, _p]),
     "mx_expert_counts": (_ci, [_p, _ci, _i64, _i64, _p, _p]),

@@ -294,7 +294,7 @@ extern "C" int mx_rmsnorm_quantize(const void *x, int x_dtype, int64_t M, int64_
                                    int64_t ldq, uint8_t *s, int64_t lds, void *stream) {
     if (M < 0 || K <= 0 || K >= (1 << 28) || !x || !dtype_ok(x_dtype) || (weight && !dtype_ok(w_dtype)) || ldx < K ||
         (out && ldo < K) || (q != nullptr) != (s != nullptr) || (q && (K % MX_BLOCK || ldq < K || lds < K / MX_BLOCK)) ||
-        (!out && !q))
+        (!out && !q && !rstd))
         return MX_EINVAL;
     if (M == 0) return MX_OK;
     const int ex = esize(x_dtype);

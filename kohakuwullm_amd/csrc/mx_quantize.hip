@@ -367,6 +367,53 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict_
     quant_tile<DUAL, R>(v, o, M, K, m0, k0, tile, tscale);
 }
 
+// RMSNorm in front of both quantizers: y = (x * rstd[row]) * w[col] in fp32 -- the two products in the order
+// rmsnorm_quant_kernel forms them, so the row-axis pair equals that kernel's bit for bit -- then the tile quantizer.
+// rstd comes from a first pass over x (mx_rmsnorm_quantize asked for nothing else); the second read of an activation
+// that fits the last-level cache is served from there.  Neither the 16-bit normalized activation nor a transposed copy
+// of it reaches memory.
+template <int DT, int WDT>
+__global__ __launch_bounds__(256) void rmsnorm_quant_dual_kernel(const void *__restrict__ x, int64_t M, int64_t K, int64_t ldx,
+                                                                  const void *__restrict__ w, const float *__restrict__ rstd,
+                                                                  QuantTileOut o) {
+    typedef TileGeom<8> G;
+    typedef typename Elem<WDT>::type TW;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[G::TK * QC_PITCH];
+    __shared__ __attribute__((aligned(4))) uint8_t tscale[G::TK * 4];
+    const int t = threadIdx.x;
+    const int64_t m0 = (int64_t)blockIdx.y * QC_TILE, k0 = (int64_t)blockIdx.x * G::TK;
+    const int64_t col = k0 + G::cg(t) * 8;
+    const int64_t row0 = m0 + G::rg(t) * 8;
+    const bool ok = col < K && m0 + (t >> 6) * 32 < M;  // K % 8 == 0 and M % 32 == 0
+    float v[8][8];
+    typename Elem<DT>::raw r[8];
+    float wv[8], rs[8];
+    if (ok) {
+        load_rows<DT, 8, false>(x, row0 * ldx + col, ldx, r);
+        const v4f r0 = *(const v4f *)(rstd + row0), r1 = *(const v4f *)(rstd + row0 + 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) rs[i] = r0[i], rs[4 + i] = r1[i];
+        if (w) {
+            Elem<WDT>::load8((const TW *)w + col, wv);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) wv[c] = 1.0f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        if (ok) {
+            Elem<DT>::unpack(r[i], v[i]);
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = w ? v[i][c] * rs[i] * wv[c] : v[i][c] * rs[i];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[i][c] = 0.0f;
+        }
+    }
+    quant_tile<true, 8>(v, o, M, K, m0, k0, tile, tscale);
+}
+
 // Several matrices behind one launch: workgroup `id` finds its matrix in the running tile
 // totals and quantizes one 128 x 128 tile of it along both axes.  For the once-per-step
 // requantization of all weight matrices of a model, where a launch per matrix (and per axis)
@@ -838,6 +885,45 @@ static int launch_cols(const void *x, int64_t M, int64_t K, int64_t ldx, uint8_t
 
 static bool cols_vec_ok(const void *x, int dt, int64_t K, int64_t ldx, const uint8_t *qT, int64_t ldqT) {
     return K % 8 == 0 && aligned(x, 16) && (ldx * esize(dt)) % 16 == 0 && aligned(qT, 16) && ldqT % 16 == 0;
+}
+
+template <int DT>
+static int launch_norm_dual(const void *x, int64_t M, int64_t K, int64_t ldx, const void *w, int w_dtype, const float *rstd,
+                            const QuantTileOut &o, hipStream_t st) {
+    dim3 grid;
+    if (!tile_grid<8>(M, K, grid)) return MX_EUNSUPPORTED;
+    switch (w ? w_dtype : (int)MX_FP32) {
+    case MX_BF16: rmsnorm_quant_dual_kernel<DT, MX_BF16><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, w, rstd, o); break;
+    case MX_FP16: rmsnorm_quant_dual_kernel<DT, MX_FP16><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, w, rstd, o); break;
+    default: rmsnorm_quant_dual_kernel<DT, MX_FP32><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, w, rstd, o); break;
+    }
+    MX_LAUNCH_CHECK();
+    return MX_OK;
+}
+
+extern "C" int mx_rmsnorm_quantize_dual(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void *weight,
+                                        int w_dtype, float eps, float *rstd, uint8_t *q, int64_t ldq, uint8_t *s,
+                                        int64_t lds, uint8_t *qT, int64_t ldqT, uint8_t *sT, int64_t ldsT, void *stream) {
+    const bool panels = stage_major(ldqT, M);
+    if (M < 0 || K <= 0 || M % MX_BLOCK || K % MX_BLOCK || !x || !rstd || !q || !s || !qT || !sT || ldx < K || ldq < K ||
+        lds < K / MX_BLOCK || (ldqT < M && !panels) || (panels && M % 128) || ldsT < M / MX_BLOCK)
+        return MX_EINVAL;
+    if (x_dtype != MX_BF16 && x_dtype != MX_FP16 && x_dtype != MX_FP32) return MX_EINVAL;
+    if (weight && w_dtype != MX_BF16 && w_dtype != MX_FP16 && w_dtype != MX_FP32) return MX_EINVAL;
+    if (M == 0) return MX_OK;
+    if (!cols_vec_ok(x, x_dtype, K, ldx, qT, ldqT) || !aligned(q, 8) || ldq % 8 || !aligned(rstd, 16) ||
+        (weight && !aligned(weight, 16)))
+        return MX_EUNSUPPORTED;
+    // first pass: the rows' reciprocal root mean squares (the row kernel, asked for nothing but rstd)
+    int rc = mx_rmsnorm_quantize(x, x_dtype, M, K, ldx, nullptr, 0, eps, nullptr, 0, rstd, nullptr, 0, nullptr, 0, stream);
+    if (rc != MX_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, 0, panels ? K * 128 : 0);
+    switch (x_dtype) {
+    case MX_BF16: return launch_norm_dual<MX_BF16>(x, M, K, ldx, weight, w_dtype, rstd, o, st);
+    case MX_FP16: return launch_norm_dual<MX_FP16>(x, M, K, ldx, weight, w_dtype, rstd, o, st);
+    default: return launch_norm_dual<MX_FP32>(x, M, K, ldx, weight, w_dtype, rstd, o, st);
+    }
 }
 
 extern "C" int mx_quantize_cols(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx, uint8_t *qT,

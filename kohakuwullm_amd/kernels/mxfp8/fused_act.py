@@ -57,3 +57,39 @@ def rmsnorm_mx(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6):
     if m and k:
         launch_rmsnorm(x2, None if weight is None else weight.contiguous(), eps, None, None, q, s)
     return q, s
+
+
+def rmsnorm_mx_dual(x: torch.Tensor, weight: torch.Tensor | None, eps: float = 1e-6, stage_major_t: bool = False):
+    """RMSNorm as both MXFP8 operands of the linear layer behind it: ``(q, s, qT, sT, rstd)``.
+
+    ``(q, s)`` ``(M,K)``, ``(M,K//32)`` is ``rmsnorm_mx(x, weight, eps)`` bit for bit (the layer's forward operand);
+    ``(qT, sT)`` ``(K,M)``, ``(K,M//32)`` is the same fp32 ``x * rstd * weight`` quantized along the tokens (the operand
+    of its weight gradient: what ``quantize_mx_cols`` would make of it); ``rstd`` ``(M,)`` fp32 is what the norm's
+    backward takes.  The normalized activation itself is never written.  ``M`` and ``K`` multiples of 32.
+    ``stage_major_t``: ``qT`` as ``(M/128, K, 128)`` panels (``M % 128 == 0``), the layout the GEMM reads fastest on long
+    token axes.  The reference has the row-axis half only (``rmsnorm_mx``, ``fused_act.py:146-175``).
+    """
+    from kohakuwullm_amd.kernels.elementwise.rmsnorm import _check
+
+    _check(x, weight, True)
+    x2 = x.contiguous().reshape(-1, x.shape[-1])
+    m, k = x2.shape
+    if m % BLOCK_SCALE or k % BLOCK_SCALE:
+        raise ValueError(f"rows={m} and K={k} must be multiples of {BLOCK_SCALE}")
+    if stage_major_t and (m % 128 or m <= 128):
+        raise ValueError(f"stage_major_t needs a multiple of 128 tokens above 128, got {m}")
+    dev, f8 = x.device, torch.float8_e4m3fn
+    q = torch.empty(m, k, device=dev, dtype=f8)
+    s = torch.empty(m, k // BLOCK_SCALE, device=dev, dtype=torch.uint8)
+    qt = torch.empty((m // 128, k, 128) if stage_major_t else (k, m), device=dev, dtype=f8)
+    st = torch.empty(k, m // BLOCK_SCALE, device=dev, dtype=torch.uint8)
+    rstd = torch.empty(m, device=dev, dtype=torch.float32)
+    if m and k:
+        w = None if weight is None else weight.contiguous()
+        _lib.invoke(
+            "mx_rmsnorm_quantize_dual", m * k * (2 * x.element_size() + 2 * (1 + 1 / BLOCK_SCALE)), x2,
+            x2.data_ptr(), _lib.MX_DTYPE[x2.dtype], m, k, x2.stride(0), 0 if w is None else w.data_ptr(),
+            0 if w is None else _lib.MX_DTYPE[w.dtype], float(eps), rstd.data_ptr(), q.data_ptr(), k, s.data_ptr(),
+            k // BLOCK_SCALE, qt.data_ptr(), 128 if stage_major_t else m, st.data_ptr(), m // BLOCK_SCALE,
+        )
+    return q, s, qt, st, rstd

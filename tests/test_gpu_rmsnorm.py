@@ -125,3 +125,56 @@ def test_backward_matches_autograd_oracle(oracle, m, k, wdtype):
     if w is not None:
         assert wd.grad.dtype == wdtype
         assert oracle.rel_error(wd.grad.cpu(), ref_dw) < 1e-2
+
+
+@pytest.mark.parametrize("m,k", [(32, 32), (64, 96), (160, 1536), (256, 2048), (384, 4096), (96, 5120)])
+@pytest.mark.parametrize("dtype,wdtype", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32), (torch.bfloat16, None)])
+def test_rmsnorm_mx_dual_matches_oracle(oracle, m, k, dtype, wdtype):
+    """Both operands of the linear layer behind the norm from one call: the row-axis pair is the oracle's
+    rms_norm_mx, the token-axis pair the oracle's column quantizer on the same fp32 normalized values (formed with
+    the oracle's rstd in the kernel's order: (x * rstd) * w, one fp32 rounding per product); the stage-major layout
+    holds the same bytes.  Rows whose rstd differs from the oracle's (an fp64 rounding on an fp32 boundary) are
+    excluded from the bit comparison as in the row-axis test; none is expected."""
+    from kohakuwullm_amd.kernels.mxfp8.fused_act import rmsnorm_mx, rmsnorm_mx_dual
+
+    x, w = _inputs(m, k, dtype, wdtype)
+    xd, wd = x.to(DEV), None if w is None else w.to(DEV)
+    q, s, qt, st, rstd = rmsnorm_mx_dual(xd, wd, 1e-6)
+    assert q.shape == (m, k) and s.shape == (m, k // 32) and qt.shape == (k, m) and st.shape == (k, m // 32)
+    rows_ok = _compare(oracle, x, w, 1e-6, None, rstd, q, s)
+    assert bool(rows_ok.all())
+    _, ref_rstd, _, _ = oracle.rms_norm_mx(x, w, 1e-6)
+    y = x.float() * ref_rstd[:, None]
+    if w is not None:
+        y = y * w.float()
+    ref_qt, ref_st = oracle.quantize_cols(y)
+    assert torch.equal(qt.view(torch.uint8).cpu(), ref_qt) and torch.equal(st.cpu(), ref_st)
+    # the same row-axis bytes as the single-axis producer
+    q1, s1 = rmsnorm_mx(xd, wd, 1e-6)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s, s1)
+    if m % 128 == 0 and m > 128:
+        _, _, panels, st2, _ = rmsnorm_mx_dual(xd, wd, 1e-6, stage_major_t=True)
+        assert panels.shape == (m // 128, k, 128) and torch.equal(st2, st)
+        assert torch.equal(panels.view(torch.uint8).permute(1, 0, 2).reshape(k, m), qt.view(torch.uint8))
+
+
+def test_rmsnorm_mx_dual_full_width_and_errors(oracle):
+    """The hidden-state matrix of the attention configuration (32768 x 2048), against the device's own single-axis
+    producer and column quantizer (bit-exact against the oracle themselves); refusals."""
+    from kohakuwullm_amd.kernels.mxfp8.fused_act import rmsnorm_mx, rmsnorm_mx_dual
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx_cols
+
+    x, w = _inputs(32768, 2048, torch.bfloat16, torch.bfloat16)
+    xd, wd = x.to(DEV), w.to(DEV)
+    q, s, qt, st, rstd = rmsnorm_mx_dual(xd, wd, 1e-6)
+    q1, s1 = rmsnorm_mx(xd, wd, 1e-6)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s, s1)
+    y = (xd.float() * rstd[:, None]) * wd.float()
+    qt1, st1 = quantize_mx_cols(y)
+    assert torch.equal(qt.view(torch.uint8), qt1.view(torch.uint8)) and torch.equal(st, st1)
+    with pytest.raises(ValueError):
+        rmsnorm_mx_dual(xd[:33], wd)  # tokens not a multiple of 32
+    with pytest.raises(ValueError):
+        rmsnorm_mx_dual(xd[:128], wd, stage_major_t=True)  # one panel is not a stage-major matrix
+    with pytest.raises(Exception):
+        rmsnorm_mx_dual(x, w)  # CPU tensors: there is no CPU path
