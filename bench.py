@@ -249,8 +249,9 @@ def _event_times(fn, iters: int, warm: int = 3):
 STREAM_KINDS = (("read", 0, 1), ("copy", 1, 2), ("triad", 2, 3), ("read2_write1", 3, 3), ("read2_write1_two_streams", 4, 3),
                 ("read3_write2", 5, 5))  # name, kind of mx_ubench_stream_cfg, bytes moved per output byte
 # launch shapes swept per mix: (threads, unroll, workgroups per CU [0: one chunk each], non-temporal bits [1 loads, 2 stores])
-STREAM_SWEEP_FULL = tuple((t, u, w, nt) for t in (256, 512, 1024) for u in (2, 4, 8) for w in (0, 8, 16, 32) for nt in (0, 1, 2, 3))
-STREAM_SWEEP_SHORT = tuple((t, u, w, nt) for t in (256, 512) for u in (4, 8) for w in (0, 16) for nt in (0, 3))
+STREAM_SWEEP_FULL = tuple((t, u, w, nt) for t in (256, 512, 1024) for u in (1, 2, 4, 8) for w in (0, 8, 16, 32) for nt in (0, 1, 2, 3))
+# the shapes that won a mix in full sweeps (one chunk per workgroup, one or two accesses in flight), and two persistent ones
+STREAM_SWEEP_SHORT = tuple((t, u, 0, nt) for t in (256, 512, 1024) for u in (1, 2) for nt in (0, 3)) + ((256, 4, 16, 3), (512, 4, 32, 3))
 STREAM_DEFAULT_POINT = (256, 4, 16, 3)  # what mx_ubench_stream runs
 
 
@@ -357,7 +358,7 @@ def measured_peaks(dev) -> dict:
         "mfma_tflops": max(short, sustained),
         "mfma_tflops_single_launch": short,
         "mfma_tflops_sustained": sustained,
-        "how": "mx_ubench_stream_cfg on 512 MiB per stream, every mix under 16 launch shapes (threads, loads in flight, grid, "
+        "how": "mx_ubench_stream_cfg on 512 MiB per stream, every mix under 14 launch shapes (threads, loads in flight, grid, "
                "non-temporal hints), best launch of the best shape; mx_ubench_mfma from registers, best single launch and the "
                "last 60 of 240 back-to-back launches; all in this run",
     }

@@ -92,6 +92,11 @@ struct Elem<MX_BF16> {
     typedef v4i raw;
     template <bool NT = false>
     static __device__ __forceinline__ raw load_raw(const void *p) { return stream_load<NT>((const v4i *)p); }
+    // value c (0..7) of a raw row chunk, converted where it is used: a kernel that keeps its tile raw holds half the registers
+    static __device__ __forceinline__ float elem(const raw &r, int c) {
+        const uint32_t w = (uint32_t)r[c >> 1];
+        return bits2f((c & 1) ? (w & 0xFFFF0000u) : (w << 16));
+    }
     static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -114,6 +119,7 @@ struct Elem<MX_FP16> {
     typedef _Float16 raw __attribute__((ext_vector_type(8)));
     template <bool NT = false>
     static __device__ __forceinline__ raw load_raw(const void *p) { return stream_load<NT>((const raw *)p); }
+    static __device__ __forceinline__ float elem(const raw &r, int c) { return (float)r[c]; }
     static __device__ __forceinline__ void unpack(const raw &r, float v[8]) {
 #pragma unroll
         for (int i = 0; i < 8; i++) v[i] = (float)r[i];

@@ -330,6 +330,91 @@ __device__ __forceinline__ void quant_tile(float (&v)[R][8], const QuantTileOut 
     __syncthreads();
 }
 
+// quant_tile<ROWS, 8, NTS> for a tile of 16-bit values kept as loaded (r[i]: row i's eight values, packed): every value
+// is converted where it is used, three times instead of once, and the thread holds 32 registers of tile instead of 64.
+// The plain row + token axis quantizer then fits 64 registers and eight waves per SIMD (90 registers and five with the
+// tile in fp32), so that the 1536 tiles of a 16384 x 1536 activation are resident at once instead of in 1.2 rounds.
+// Same arithmetic on the same values: bit-identical outputs.
+template <int DT, bool ROWS, bool NTS>
+__device__ __forceinline__ void quant_tile_raw(typename Elem<DT>::raw (&r)[8], bool ok, const QuantTileOut &o, int64_t M,
+                                               int64_t K, int64_t m0, int64_t kc0, uint8_t *tile, uint8_t *tscale) {
+    typedef TileGeom<8> G;
+    typedef Elem<DT> E;
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int cg = G::cg(t), rg = G::rg(t);
+    const int64_t col = kc0 + cg * 8;
+    const int64_t row0 = m0 + rg * 8;
+    auto val = [&](int i, int c) { return ok ? E::elem(r[i], c) : 0.0f; };
+
+    if (ROWS) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float v[8];
+#pragma unroll
+            for (int c = 0; c < 8; c++) v[c] = val(i, c);
+            const float amax = quad_max(amax8(v));
+            const uint32_t byte = scale_byte(amax);
+            const float inv = inv_scale(byte);
+            const uint32_t packed = gather_row_scales(byte, lane);
+            if (ok) {
+                v2i codes;
+                codes[0] = (int)pack4_e4m3(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+                codes[1] = (int)pack4_e4m3(v[4] * inv, v[5] * inv, v[6] * inv, v[7] * inv);
+                stream_store<NTS>((v2i *)(o.q + (o.q_ks ? (col >> 7) * o.q_ks + (row0 + i) * 128 + (col & 127) : (row0 + i) * o.ldq + col)), codes);
+                uint8_t *sp = o.s + (row0 + i) * o.lds + (col >> 5);
+                const bool full = kc0 + G::TK <= K;
+                if (o.pack_row_scales && full) {
+                    if (cg == 0) *(uint32_t *)sp = packed;
+                } else if ((cg & 3) == 0) {
+                    *sp = (uint8_t)byte;
+                }
+            }
+        }
+    }
+    // The column pass converts the raw values again.  Without this the compiler keeps the 64 conversions of the row
+    // pass alive for it, which is the register cost this function exists to avoid.
+#pragma unroll
+    for (int i = 0; i < 8; i++) asm volatile("" : "+v"(r[i]));
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = val(i, c);
+        float cm = amax8(v);
+        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        const uint32_t byte = scale_byte(cm);
+        const float inv = inv_scale(byte);
+        v2i codes;
+        codes[0] = (int)pack4_e4m3(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+        codes[1] = (int)pack4_e4m3(v[4] * inv, v[5] * inv, v[6] * inv, v[7] * inv);
+        *(v2i *)(tile + (cg * 8 + c) * QC_PITCH + rg * 8) = codes;
+        if ((rg & 3) == 0) tscale[(cg * 8 + c) * 4 + wave] = (uint8_t)byte;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < G::TK / 32; j++) {
+        const int kr = j * 32 + (t >> 3), ch = t & 7;
+        if (kc0 + kr < K && m0 + ch * 16 < M) {
+            const v2i *src = (const v2i *)(tile + kr * QC_PITCH + ch * 16);
+            const v2i a = src[0], b = src[1];
+            stream_store<NTS>((v4i *)(o.qT + (o.qT_ks ? (m0 >> 7) * o.qT_ks + (kc0 + kr) * 128 : (kc0 + kr) * o.ldqT + m0) + ch * 16),
+                              v4i{a[0], a[1], b[0], b[1]});
+        }
+    }
+    if (t < G::TK && kc0 + t < K) {
+        uint8_t *sp = o.sT + (kc0 + t) * o.ldsT + (m0 >> 5);
+        const int64_t nb = (M - m0) >> 5;
+        if (o.pack_col_scales && nb >= 4) {
+            *(uint32_t *)sp = *(const uint32_t *)(tscale + t * 4);
+        } else {
+            for (int b = 0; b < 4 && b < nb; b++) sp[b] = tscale[t * 4 + b];
+        }
+    }
+    __syncthreads();
+}
+
 // Loads the thread's R rows of 8 values of one operand raw (all loads in flight before any conversion).
 template <int DT, int R, bool NT>
 __device__ __forceinline__ void load_rows(const void *x, int64_t first, int64_t ld, typename Elem<DT>::raw (&r)[R]) {
@@ -338,7 +423,8 @@ __device__ __forceinline__ void load_rows(const void *x, int64_t first, int64_t 
     for (int i = 0; i < R; i++) r[i] = Elem<DT>::template load_raw<NT>((const T *)x + first + i * ld);
 }
 
-template <int DT, bool DUAL, int R>
+// RAW (16-bit inputs, R = 8): the tile stays packed as loaded (quant_tile_raw): 64 registers, eight waves per SIMD.
+template <int DT, bool DUAL, int R, bool RAW = false>
 __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict__ x, int64_t M, int64_t K, int64_t ldx,
                                                           QuantTileOut o) {
     typedef TileGeom<R> G;
@@ -349,12 +435,17 @@ __global__ __launch_bounds__(256) void quant_cols_kernel(const void *__restrict_
     const int64_t col = k0 + G::cg(t) * 8;
     const int64_t row0 = m0 + G::rg(t) * R;
     const bool ok = col < K && m0 + (t >> 6) * 32 < M;  // K % 8 == 0 and M % 32 == 0
-    float v[R][8];
     // the thread's loads go out together (row by row, each waited for the one before it)
     typename Elem<DT>::raw r[R];
     // both axes at once is the activation path of a training step, where the 16-bit input is not read again soon: its
     // loads carry the non-temporal hint; the codes are read by the next GEMM and are stored plainly
     if (ok) load_rows<DT, R, DUAL>(x, row0 * ldx + col, ldx, r);
+    if constexpr (RAW) {
+        static_assert(DT != MX_FP32 && R == 8, "a packed tile of 16-bit values");
+        quant_tile_raw<DT, DUAL, false>(r, ok, o, M, K, m0, k0, tile, tscale);
+        return;
+    }
+    float v[R][8];
 #pragma unroll
     for (int i = 0; i < R; i++) {
         if (ok) {
@@ -877,8 +968,16 @@ static int launch_cols(const void *x, int64_t M, int64_t K, int64_t ldx, uint8_t
                        int64_t ldsT, uint8_t *q, int64_t ldq, uint8_t *s, int64_t lds, hipStream_t st, int64_t qT_ks = 0) {
     dim3 grid;
     if (!tile_grid<MX_QR_COLS>(M, K, grid)) return MX_EUNSUPPORTED;
-    quant_cols_kernel<DT, DUAL, MX_QR_COLS><<<grid, dim3(256), 0, st>>>(x, M, K, ldx,
-                                                                         tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, 0, qT_ks));
+    const QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, q, ldq, s, lds, 0, qT_ks);
+    // Both axes of a 16-bit matrix whose tiles are all resident at once with eight waves per SIMD, but not with the five
+    // the fp32 tile allows, go to the packed-tile kernel: 16384 x 1536 (1536 tiles on 256 CUs) 27.0 -> 24.9 us.  Larger
+    // matrices run several rounds either way and are faster with fewer, fatter waves (16384 x 4096: 54.4 against 58.9 us).
+    bool raw = false;
+    if constexpr (DT != MX_FP32 && DUAL) raw = (int64_t)grid.x * grid.y <= 8 * (int64_t)num_cus();
+    if constexpr (DT != MX_FP32 && DUAL) {
+        if (raw) quant_cols_kernel<DT, DUAL, MX_QR_COLS, true><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, o);
+    }
+    if (!raw) quant_cols_kernel<DT, DUAL, MX_QR_COLS><<<grid, dim3(256), 0, st>>>(x, M, K, ldx, o);
     MX_LAUNCH_CHECK();
     return MX_OK;
 }
