@@ -288,6 +288,48 @@ def measure_stream(dev, out_bytes: int = 1 << 29, iters: int = 10, sweep=STREAM_
     return out
 
 
+def measure_tile_patterns(dev, iters: int = 12) -> dict:
+    """Microseconds the access pattern of the 128 x 128 tile quantizers takes WITHOUT their arithmetic
+    (mx_ubench_tile_pattern), at the shapes of the feed-forward step's three bandwidth kernels: the same bytes read
+    from and written to the same places, on inputs that rotate through more than the last-level cache holds; best
+    over the hint and layout choices.  A kernel cannot be faster than its own pattern."""
+    import torch
+
+    from kohakuwullm_amd import _lib
+
+    lib = _lib.load()
+    st = torch.cuda.current_stream(dev).cuda_stream
+    sets = 3
+    out = {}
+    for entry, inputs, cols in (("mx_quantize_dual", 1, DIM), ("mx_swiglu_quantize_dual", 2, FFN), ("mx_swiglu_bwd_quantize_dual", 3, FFN)):
+        width = cols * (2 if inputs >= 2 else 1)
+        xs = [torch.empty(TOKENS, width, dtype=torch.bfloat16, device=dev).normal_() for _ in range(sets)]
+        ys = [torch.empty(TOKENS, cols, dtype=torch.bfloat16, device=dev).normal_() for _ in range(sets)] if inputs == 3 else None
+        outs = [[torch.empty(TOKENS * cols, dtype=torch.uint8, device=dev) for _ in range(4 if inputs == 3 else 2)] for _ in range(sets)]
+        best = None
+        for nt in (0, 1, 3):
+            for panels in (0, 1):
+                state = {"i": 0}
+
+                def call():
+                    i = state["i"] % sets
+                    state["i"] += 1
+                    o = outs[i]
+                    _lib.check(lib.mx_ubench_tile_pattern(inputs, 1, nt, panels, xs[i].data_ptr(), width, ys[i].data_ptr() if ys else None,
+                                                          TOKENS, cols, o[0].data_ptr(), o[1].data_ptr(),
+                                                          o[2].data_ptr() if inputs == 3 else None, o[3].data_ptr() if inputs == 3 else None,
+                                                          st), "mx_ubench_tile_pattern")
+
+                ts = _event_times(call, iters, warm=sets)
+                med = ts[len(ts) // 2] * 1e3
+                if best is None or med < best["us_median"]:
+                    best = {"us_median": round(med, 1), "nontemporal": nt, "stage_major": bool(panels),
+                            "gbs": round(TOKENS * cols * (2 * inputs + (4 if inputs == 3 else 2)) / med / 1e3, 1)}
+        out[entry] = best
+        del xs, ys, outs
+    return out
+
+
 def measure_mfma(dev, iters: int = 4000, repeats: int = 5) -> dict:
     """Issue rate of the block-scaled fp8 MFMA from registers in TFLOP/s: both tile shapes, zero and hashed operands."""
     import torch
@@ -914,10 +956,14 @@ def main() -> None:
     peaks = measured_peaks(dev)
     # every bandwidth launch against the best streaming rate measured for its own read : write mix
     mix_of = {"mx_quantize_dual": "hbm_copy_gbs", "mx_swiglu_bwd_quantize_dual": "hbm_read3_write2_gbs"}
+    patterns = measure_tile_patterns(dev) if args.workload == "ffn" else {}
     for row in launches:
         if row["unit"] == "GB/s":
             row["mix_ceiling"] = peaks[mix_of.get(row["entry"], "hbm_read2_write1_gbs")]
             row["frac_of_mix_ceiling"] = round(row["rate_median"] / row["mix_ceiling"], 4)
+            if row["entry"] in patterns:  # the kernel's own access pattern without arithmetic: a tighter bound
+                row["access_pattern_us"] = patterns[row["entry"]]["us_median"]
+                row["frac_of_access_pattern"] = round(row["access_pattern_us"] / row["us_median"], 4)
 
     out = {
         "metric": "MXFP8 linear fwd+bwd TFLOP/s (quantizers included)",
@@ -968,6 +1014,7 @@ def main() -> None:
             "share_of_step": round(quant_ms / (quant_ms + gemm_ms), 4),
         },
         "peaks_measured": peaks,
+        "tile_access_patterns": patterns,
         "weight_refresh_ms": round(weight_refresh_ms, 4),
         "launch_breakdown": launches,
     }

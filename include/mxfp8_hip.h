@@ -509,6 +509,20 @@ int mx_ubench_stream_cfg(int kind, int threads, int unroll, int wgs_per_cu, int 
                          const void *b, void *c, int64_t out_bytes, void *stream);
 
 /*
+ * The memory access pattern of the 128 x 128 tile quantizers without their arithmetic, as a second, tighter ceiling
+ * for them: every 256-thread workgroup reads a tile of `inputs` 16-bit matrices the way those kernels do (1: x (M,K),
+ * pitch ldx; 2: the halves x[:, :K] and x[:, K:2K] of a (M,2K) matrix; 3: those and y (M,K)), writes 8 bytes per
+ * 16 read into q (M,K) bytes and, with transposed != 0, the transposed byte tile into qT (K,M) (inputs == 3: a
+ * second pair q2, qT2, as the SwiGLU' quantizer has two output halves).  panels != 0: q and qT in the stage-major
+ * layout of mx_quantize_dual.  nontemporal as in mx_ubench_stream_cfg.  M % 128 == 0, K % 128 == 0.  The values
+ * written are a fold of the values read, nothing more.
+ * Same rule of the reference as mx_ubench_stream (src/kohakuwullm/bench/core/timing.py:231-268).
+ */
+int mx_ubench_tile_pattern(int inputs, int transposed, int nontemporal, int panels, const void *x, int64_t ldx,
+                           const void *y, int64_t M, int64_t K, uint8_t *q, uint8_t *qT, uint8_t *q2, uint8_t *qT2,
+                           void *stream);
+
+/*
  * Register-resident loop of the block-scaled fp8 MFMA (bit 0 of wide clear: v_mfma_scale_f32_16x16x128_f8f6f4
  * with 8 independent accumulator tiles per wave, set: ..._32x32x64_... with 4), 8 waves on every CU (bit 1 of
  * wide set: 4 waves, one per SIMD; bit 2 set, 16x16x128 form only: scale bytes come from vector registers instead

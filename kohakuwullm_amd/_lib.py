@@ -73,6 +73,7 @@ SIGNATURES = {
     "mx_gemm_nt_batch": (_ci, [_p, _ci, _ci, _p, _i64, _p]),
     "mx_ubench_stream": (_ci, [_ci, _p, _p, _p, _i64, _p]),
     "mx_ubench_stream_cfg": (_ci, [_ci, _ci, _ci, _ci, _ci, _p, _p, _p, _i64, _p]),
+    "mx_ubench_tile_pattern": (_ci, [_ci, _ci, _ci, _ci, _p, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p]),
     "mx_ubench_mfma": (_i64, [_ci, _ci, _ci, _p, _i64, _p]),
 }
 

@@ -108,6 +108,60 @@ static int launch_stream_unroll(int unroll, bool ntl, bool nts, dim3 grid, dim3 
     return MX_OK;
 }
 
+// The memory access pattern of the 128 x 128 tile quantizers without their arithmetic: 256 threads, thread (t % 16,
+// t / 16) reads 16 bytes of each of 8 rows (a row pitch apart) from every input, writes 8 bytes per row into a (M, K)
+// byte matrix (the row-axis codes' place) and, through LDS, the transposed byte tile into a (K, M) byte matrix in
+// 16-byte pieces (row-major, or 128-token panels: the stage-major layout).  INPUTS 1: one 16-bit matrix (the plain
+// quantizers), 2: the two halves of a (M, 2K) matrix (SwiGLU), 3: those and a (M, K) matrix, two sets of outputs
+// (SwiGLU').  What this reaches bounds what those kernels can: the same bytes in the same places, no arithmetic.
+template <int INPUTS, bool TRANSPOSED, bool NTL, bool NTS>
+__global__ __launch_bounds__(256) void tile_pattern_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ y,
+                                                            int64_t M, int64_t K, int64_t ldx, uint8_t *__restrict__ q,
+                                                            uint8_t *__restrict__ qT, uint8_t *__restrict__ q2,
+                                                            uint8_t *__restrict__ qT2, int panels) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 136];
+    const int t = threadIdx.x, cg = t & 15, rg = t >> 4;
+    const int64_t m0 = (int64_t)blockIdx.y * 128, k0 = (int64_t)blockIdx.x * 128;
+    const int64_t col = k0 + cg * 8, row0 = m0 + rg * 8;
+    v4i a[8], b[8], c[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        a[i] = ld16<NTL>((const v4i *)(x + (row0 + i) * ldx + col));
+        if (INPUTS >= 2) b[i] = ld16<NTL>((const v4i *)(x + (row0 + i) * ldx + K + col));
+        if (INPUTS == 3) c[i] = ld16<NTL>((const v4i *)(y + (row0 + i) * K + col));
+    }
+#pragma unroll
+    for (int pass = 0; pass < (INPUTS == 3 ? 2 : 1); pass++) {
+        uint8_t *qq = pass ? q2 : q, *qqT = pass ? qT2 : qT;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            v4i v = a[i];
+            if (INPUTS >= 2) v ^= pass ? c[i] : b[i];
+            if (INPUTS == 3 && !pass) v ^= c[i];
+            typedef int v2i_t __attribute__((ext_vector_type(2)));
+            const v2i_t codes = {v[0] ^ v[1], v[2] ^ v[3]};
+            v2i_t *dst = (v2i_t *)(qq + (panels ? (col >> 7) * (M * 128) + (row0 + i) * 128 + (col & 127) : (row0 + i) * K + col));
+            if (NTS) __builtin_nontemporal_store(codes, dst);
+            else *dst = codes;
+            if (TRANSPOSED) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) tile[(cg * 8 + e) * 136 + rg * 8 + i] = (uint8_t)(v[e >> 1] >> ((e & 1) * 16));
+            }
+        }
+        if (TRANSPOSED) {
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int kr = j * 32 + (t >> 3), ch = t & 7;
+                const int *src = (const int *)(tile + kr * 136 + ch * 16);
+                st16<NTS>((v4i *)(qqT + (panels ? (m0 >> 7) * (K * 128) + (k0 + kr) * 128 : (k0 + kr) * M + m0) + ch * 16),
+                          v4i{src[0], src[1], src[2], src[3]});
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // Register-resident block-scaled fp8 MFMA loop: ACCS independent accumulator tiles per wave, operands that never
 // change, no memory traffic.  `random` fills the operand registers with a per-lane hash (switching activity of
 // real data) instead of zeros: the part's clock, and with it this peak, depends on what the multipliers see.
@@ -199,6 +253,40 @@ extern "C" int mx_ubench_stream_cfg(int kind, int threads, int unroll, int wgs_p
     default: rc = launch_stream_unroll<5>(unroll, ntl, nts, grid, block, st, pa, pb, pc, n); break;
     }
     if (rc != MX_OK) return rc;
+    return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
+}
+
+template <int INPUTS, bool TRANSPOSED>
+static void launch_tile_pattern(int nt, dim3 grid, hipStream_t st, const uint16_t *x, const uint16_t *y, int64_t M, int64_t K,
+                                int64_t ldx, uint8_t *q, uint8_t *qT, uint8_t *q2, uint8_t *qT2, int panels) {
+    const dim3 block(256);
+    switch (nt) {
+    case 0: tile_pattern_kernel<INPUTS, TRANSPOSED, false, false><<<grid, block, 0, st>>>(x, y, M, K, ldx, q, qT, q2, qT2, panels); break;
+    case 1: tile_pattern_kernel<INPUTS, TRANSPOSED, true, false><<<grid, block, 0, st>>>(x, y, M, K, ldx, q, qT, q2, qT2, panels); break;
+    case 2: tile_pattern_kernel<INPUTS, TRANSPOSED, false, true><<<grid, block, 0, st>>>(x, y, M, K, ldx, q, qT, q2, qT2, panels); break;
+    default: tile_pattern_kernel<INPUTS, TRANSPOSED, true, true><<<grid, block, 0, st>>>(x, y, M, K, ldx, q, qT, q2, qT2, panels); break;
+    }
+}
+
+extern "C" int mx_ubench_tile_pattern(int inputs, int transposed, int nontemporal, int panels, const void *x, int64_t ldx,
+                                      const void *y, int64_t M, int64_t K, uint8_t *q, uint8_t *qT, uint8_t *q2, uint8_t *qT2,
+                                      void *stream) {
+    if (inputs < 1 || inputs > 3 || nontemporal < 0 || nontemporal > 3 || M <= 0 || K <= 0 || M % 128 || K % 128) return MX_EINVAL;
+    if (!x || !q || (transposed && !qT) || (inputs == 3 && (!y || !q2 || (transposed && !qT2)))) return MX_EINVAL;
+    if (ldx < (inputs >= 2 ? 2 * K : K) || ldx % 8 || ((uintptr_t)x & 15) || ((uintptr_t)y & 15) || ((uintptr_t)q & 15) ||
+        ((uintptr_t)qT & 15) || ((uintptr_t)q2 & 15) || ((uintptr_t)qT2 & 15) || M / 128 > 65535)
+        return MX_EINVAL;
+    hipStream_t st = (hipStream_t)stream;
+    if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
+    const dim3 grid((unsigned)(K / 128), (unsigned)(M / 128));
+    const uint16_t *px = (const uint16_t *)x, *py = (const uint16_t *)y;
+    const int p = panels ? 1 : 0;
+    if (inputs == 1 && transposed) launch_tile_pattern<1, true>(nontemporal, grid, st, px, py, M, K, ldx, q, qT, q2, qT2, p);
+    else if (inputs == 1) launch_tile_pattern<1, false>(nontemporal, grid, st, px, py, M, K, ldx, q, qT, q2, qT2, p);
+    else if (inputs == 2 && transposed) launch_tile_pattern<2, true>(nontemporal, grid, st, px, py, M, K, ldx, q, qT, q2, qT2, p);
+    else if (inputs == 2) launch_tile_pattern<2, false>(nontemporal, grid, st, px, py, M, K, ldx, q, qT, q2, qT2, p);
+    else if (transposed) launch_tile_pattern<3, true>(nontemporal, grid, st, px, py, M, K, ldx, q, qT, q2, qT2, p);
+    else launch_tile_pattern<3, false>(nontemporal, grid, st, px, py, M, K, ldx, q, qT, q2, qT2, p);
     return hipGetLastError() == hipSuccess ? MX_OK : MX_ELAUNCH;
 }
 
