@@ -407,8 +407,8 @@ def measured_peaks(dev) -> dict:
 
 # Bytes the GEMM launches of one step move between the L2s and the fabric, per launch, from the
 # FETCH_SIZE and WRITE_SIZE counter runs summarised under profiles/ (each scaled by what the
-# counter reads for a device copy of known size): 2054 MiB over 4 launches.
-GEMM_TRAFFIC_PER_LAUNCH = {"ffn": 514 * 2**20}
+# counter reads for a device copy of known size): 2049 MiB over 4 launches.
+GEMM_TRAFFIC_PER_LAUNCH = {"ffn": 512 * 2**20}
 TRAFFIC_SOURCE = ("a constant, not measured in this run: the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in "
                   "profiles/gemm_nt_kernel_dense_ffn_fwd_bwd.md")
 
