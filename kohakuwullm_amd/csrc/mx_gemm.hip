@@ -197,20 +197,6 @@ struct DenseProblem {
                 for (int j = 0; j < S::NT; j++) dst[(i * S::NT + j) * S::NTHR + L.tid] = acc[i][j];
             return -1;
         }
-#ifdef MX_BURN
-        // timing experiment only: MX_BURN dependent VALU instructions per output value in front of the stores
-#pragma unroll
-        for (int i = 0; i < S::MT; i++)
-#pragma unroll
-            for (int j = 0; j < S::NT; j++)
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    float x = acc[i][j][v];
-#pragma unroll
-                    for (int r = 0; r < MX_BURN; r++) asm volatile("v_fma_f32 %0, %0, %0, %0" : "+v"(x));
-                    acc[i][j][v] = x;
-                }
-#endif
         // Interior tiles of a vector-aligned C store unconditionally: every lane issues NST stores.
         const bool interior = t.m0 + S::BM <= p.M && t.n0 + S::BN <= p.N && p.c_vec && !p.accumulate;
         // component v of a lane's NT sub-tiles (i, 0..NT-1): row 16 i + 4 g + v, NT consecutive N from NT r16
