@@ -536,66 +536,91 @@ struct GroupedProblem {
         const bool tok = p.htq != nullptr;
         uint32_t keep[2][S::MT][4][4];  // [gate | value][slab][row][pair of columns]
         const int H = p.N;
-        const int hblock = t.n0 + L.wn * S::WTN + 32 * (L.r16 >> 2);  // the 32 hidden units of a quad
-        const int h = t.n0 + L.wn * S::WTN + 8 * L.r16;
+        // Lane-dependent offsets are derived from an opaque copy of the lane id.  From the plain one they are
+        // invariants of the tile loop: the compiler computes them once (sixteen row numbers alone), cannot keep them
+        // in registers across the main loop, and reloads each from scratch memory right before its use behind a full
+        // vector-memory wait -- which also waits for every load and store in flight.
+        const Lane Lo = opaque(L);
+        const int o_tid = Lo.tid, o_r16 = Lo.lane & 15, o_g = Lo.lane >> 4;
+        const int hblock = t.n0 + L.wn * S::WTN + 32 * (o_r16 >> 2);  // the 32 hidden units of a quad
+        const int h = t.n0 + L.wn * S::WTN + 8 * o_r16;
         const bool col_ok = hblock < H;
+        auto row_at = [&](int i, int v) { return t.row0 + L.wm * S::WTM + 16 * i + 4 * o_g + v; };
+        // Row metadata once per tile: lane l of a wave fetches the pair index and the gate factor of the wave's row l
+        // (two dependent loads per tile); a step takes its rows' values from those lanes.  Fetched per slab of rows by
+        // the lanes that use them, the chain order -> gate cost two memory round trips per slab.
+        const int meta_m = t.row0 + L.wm * S::WTM + (Lo.lane < S::WTM ? Lo.lane : S::WTM - 1);
+        const int pair_l = p.order[meta_m < t.end ? meta_m : t.end - 1];
+        asm volatile("" ::: "memory");  // the first step's requests go out behind this load, not behind the chain's second
+        // The rows of a lane are taken RS at a time, and what a step reads from memory -- the fp8 copy of h, its scale
+        // byte, the stored pre -- is requested one step ahead, in front of the previous step's arithmetic and stores.
+        // Vector memory operations retire in order: loads issued behind a step's stores would wait for those stores
+        // to reach the L2, and all eight waves of the workgroup would then sit through a memory round trip per step
+        // with nothing to issue.  The compiler barriers keep the order written here.
+        constexpr int RS = 1, STEPS = S::MT * 4 / RS;  // more rows per step, or requests further ahead, spill and are slower
+        struct StepLoads {
+            v2i hc[RS];
+            uint32_t hsb[RS];
+            v4i pg[RS], pv[RS];
+        };
+        const int hh = col_ok ? h : 0, hb = col_ok ? hblock : 0;  // clamped: loaded, never used
+        auto request = [&](int s, StepLoads &d) {
 #pragma unroll
-        for (int i = 0; i < S::MT; i++) {
-            int pair[4];
-            float gate[4];
-            v2i hc[4];
-            uint32_t hsb[4];
-            v4i pg[4], pv[4];
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int m = row_of(t, L, i, v);
+            for (int vv = 0; vv < RS; vv++) {
+                const int m = row_at(s * RS / 4, s * RS % 4 + vv);
                 const int mm = m < t.end ? m : t.end - 1;
-                pair[v] = p.order[mm];
-                const int hh = col_ok ? h : 0, hb = col_ok ? hblock : 0;  // clamped: loaded, never used
-                hc[v] = *(const v2i *)(p.hq + (int64_t)mm * p.ldhq + hh);
-                hsb[v] = p.hs[(int64_t)mm * p.ldhs + (hb >> 5)];
+                d.hc[vv] = *(const v2i *)(p.hq + (int64_t)mm * p.ldhq + hh);
+                d.hsb[vv] = p.hs[(int64_t)mm * p.ldhs + (hb >> 5)];
                 const uint16_t *pp = (const uint16_t *)p.pre + (int64_t)mm * p.ldpre + hh;
-                pg[v] = *(const v4i *)pp;
-                pv[v] = *(const v4i *)(pp + H);
+                d.pg[vv] = *(const v4i *)pp;
+                d.pv[vv] = *(const v4i *)(pp + H);
             }
-            // The four gate loads go out together and are converted afterwards.  (With the dtype test and
-            // the conversion inside the loop the compiler issued them one at a time, each behind a full
-            // wait for the one before: five memory latencies per slab of rows instead of two.)
-            if (p.gate_f32) {
+        };
+        constexpr int AHEAD = 1;
+        StepLoads buf[AHEAD + 1];
 #pragma unroll
-                for (int v = 0; v < 4; v++) gate[v] = ((const float *)p.gate)[pair[v]];
-            } else {
-                uint16_t raw[4];
+        for (int s = 0; s < AHEAD; s++) request(s, buf[s]);
+        asm volatile("" ::: "memory");
+        float gate_l;
+        if (p.gate_f32) {
+            gate_l = ((const float *)p.gate)[pair_l];
+        } else {
+            const uint16_t raw = ((const uint16_t *)p.gate)[pair_l];
+            gate_l = CDT == MX_BF16 ? bits2f((uint32_t)raw << 16) : (float)__builtin_bit_cast(_Float16, raw);
+        }
 #pragma unroll
-                for (int v = 0; v < 4; v++) raw[v] = ((const uint16_t *)p.gate)[pair[v]];
+        for (int s = 0; s < STEPS; s++) {
+            if (s + AHEAD < STEPS) request(s + AHEAD, buf[(s + AHEAD) % (AHEAD + 1)]);
+            asm volatile("" ::: "memory");
+            const StepLoads &d = buf[s % (AHEAD + 1)];
 #pragma unroll
-                for (int v = 0; v < 4; v++)
-                    gate[v] = CDT == MX_BF16 ? bits2f((uint32_t)raw[v] << 16) : (float)__builtin_bit_cast(_Float16, raw[v]);
-            }
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int m = row_of(t, L, i, v);
+            for (int vv = 0; vv < RS; vv++) {
+                const int i = s * RS / 4, v = s * RS % 4 + vv;
+                const int m = row_at(i, v);
                 const bool row_ok = m < t.end;
                 const bool ok = row_ok && col_ok;
+                const int src = 16 * i + 4 * o_g + v;  // the lane of this wave that holds row (i, g, v)'s metadata
+                const int pair = __shfl(pair_l, src, 64);
+                const float gate = __shfl(gate_l, src, 64);
                 float a[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) a[e] = acc[i][e][v];
                 float dg[8], dv[8], dot = 0.0f;
                 if (ok) {
                     // h read back from its fp8 copy: the forward multiplied those values
-                    const float hscale = bits2f(hsb[v] << 23);
+                    const float hscale = bits2f(d.hsb[vv] << 23);
                     float gq[8], vq[8];
-                    unpack8<CDT>(pg[v], gq);
-                    unpack8<CDT>(pv[v], vq);
+                    unpack8<CDT>(d.pg[vv], gq);
+                    unpack8<CDT>(d.pv[vv], vq);
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
                         typedef float v2f __attribute__((ext_vector_type(2)));
-                        const int word = hc[v][e >> 2];
+                        const int word = d.hc[vv][e >> 2];
                         const v2f pairv = (e & 2) ? __builtin_amdgcn_cvt_pk_f32_fp8(word, true)
                                                   : __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
                         dot += a[e] * pairv[e & 1];  // times the block's power-of-two scale once, below (exact)
                         const float sg = sigmoid_f(gq[e]);
-                        const float dhs = a[e] * gate[v] * sg;
+                        const float dhs = a[e] * gate * sg;
                         dg[e] = dhs * vq[e] * (1.0f + gq[e] * (1.0f - sg));
                         dv[e] = dhs * gq[e];
                     }
@@ -634,7 +659,7 @@ struct GroupedProblem {
                     uint8_t *qp = p.dpq + (int64_t)m * p.lddpq + h;
                     *(v2i *)qp = cg;
                     *(v2i *)(qp + H) = cv;
-                    if ((L.r16 & 3) == 0) {
+                    if ((o_r16 & 3) == 0) {
                         uint8_t *sp = p.dps + (int64_t)m * p.lddps + (hblock >> 5);
                         sp[0] = (uint8_t)bg;
                         sp[H >> 5] = (uint8_t)bv;
@@ -645,8 +670,9 @@ struct GroupedProblem {
                 }
                 // the dot product over the expert width is split across lanes, waves and N tiles
                 dot = row16_sum(dot);
-                if (row_ok && L.r16 == 0) atomicAdd(p.dgate + pair[v], dot);
+                if (row_ok && o_r16 == 0) atomicAdd(p.dgate + pair, dot);
             }
+            asm volatile("" ::: "memory");
         }
         if (!tok) return -1;
 
@@ -658,8 +684,6 @@ struct GroupedProblem {
         // memory right before its use behind a full vector-memory wait, which also waited for the
         // pass's previous global store: the stores of a pass went out one round trip at a time
         // (127 reloads per tile; C4: 235 -> 224 us).
-        const Lane Lo = opaque(L);
-        const int o_tid = Lo.tid, o_r16 = Lo.lane & 15, o_g = Lo.lane >> 4;
 #pragma unroll
         for (int pass = 0; pass < 4; pass++) {
             // pass = (gate | value, low | high four of the lane's eight columns); staged column
