@@ -888,6 +888,9 @@ def main() -> None:
         if gflop:
             sampled["value_at_median"] = round(gflop / ts[len(ts) // 2], 2)
     sampled.update(settled)
+    # device memory held at the high-water mark of the steps so far (inputs, weights, caches, one step's activations and
+    # the K-split workspace of the GEMM wrappers), before the microbenchmarks below allocate their own buffers
+    sampled["peak_memory_mib"] = round(torch.cuda.max_memory_allocated(dev) / 2**20, 1)
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)

@@ -786,16 +786,31 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t *__restrict
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) acc[e] = 0.0f;
-    for (int k = 0; k < top_k; k++) {
-        const int64_t pair = t * top_k + k;
-        const int pos = inv[pair];
-        if (pos < 0) continue;
-        float scale = 1.0f;
-        if (gate) scale = gate_f32 ? ((const float *)gate)[pair] : load_act<CDT>(gate, pair);
-        float v[8];
-        unpack8<CDT>(*(const v4i *)(y + (int64_t)pos * ldy + c), v);
+    // Eight slots at a time: their positions and gate factors first, then all their rows, then the sums in slot order.
+    // One slot after the other, every slot waited for its position and then for its row: two memory round trips
+    // per slot in a kernel that does nothing else (61 -> 47 us for six slots per token at the benchmark's routing).
+    for (int k0 = 0; k0 < top_k; k0 += 8) {
+        int pos[8];
+        float scale[8];
+        v4i row[8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] += scale * v[e];
+        for (int k = 0; k < 8; k++) {
+            const int64_t pair = t * top_k + k0 + k;
+            pos[k] = k0 + k < top_k ? inv[pair] : -1;
+            scale[k] = 1.0f;
+            if (gate && k0 + k < top_k) scale[k] = gate_f32 ? ((const float *)gate)[pair] : load_act<CDT>(gate, pair);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if (pos[k] >= 0) row[k] = *(const v4i *)(y + (int64_t)pos[k] * ldy + c);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            if (pos[k] < 0) continue;
+            float v[8];
+            unpack8<CDT>(row[k], v);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] += scale[k] * v[e];
+        }
     }
     uint32_t w[4];
 #pragma unroll

@@ -30,6 +30,13 @@ from kohakuwullm_amd.kernels.mxfp8.quantize import (
 
 _FP8 = torch.float8_e4m3fn
 
+# The two projection outputs that only the SwiGLU quantizers read (`gu`, `dh`) are allocated with 128 spare
+# elements per row.  Their natural pitches (16 KiB and 8 KiB at the benchmark shape) put the 128 rows a quantizer
+# tile reads at once on a few memory channels; 256 bytes more spread them.  Measured in the step at 16384 x 1536 x
+# 4096: SwiGLU 75.6 -> 73.1 us, SwiGLU' 135.0 -> 129.4 us, the GEMM that writes `gu` 183.7 -> 186.0 us (64 or 256
+# elements: no gain).
+_PITCH_PAD = 128
+
 
 def swiglu_mx_dual(gu: torch.Tensor, stage_major_t: bool = False):
     """``h = silu(gu[:, :H]) * gu[:, H:]`` as ``(q, s, qT, sT)``: blocks along H and along tokens.
@@ -132,7 +139,7 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         # GEMM, then one bandwidth-bound pass for SwiGLU and both casts: measured faster at the
         # benchmark shape (220 + 89 us) than the same work in the GEMM's epilogue
         # (fused_swiglu_projection: 329 us), whose vector ALU work cannot overlap the MFMAs.
-        gu = mxfp8_matmul_pq(xq, xs, *in_f, compute)
+        gu = mxfp8_matmul_pq(xq, xs, *in_f, compute, out_pad=_PITCH_PAD)
         hq, hs, htq, hts = swiglu_mx_dual(gu, stage_major_t=sm)
         y = mxfp8_matmul_pq(hq, hs, *out_f, compute)
         if any(ctx.needs_input_grad):
@@ -149,7 +156,7 @@ class _MXFP8SwiGLUMLP(torch.autograd.Function):
         d2d = dout.reshape(-1, shape[-1]).to(ctx.compute).contiguous()
         tokens = d2d.shape[0]
         dq, ds, dtq, dts = quantize_mx_dual(pad_tokens(d2d), stage_major_t=ctx.stage_major)
-        dh = mxfp8_matmul_pq(dq, ds, wout_dq, wout_ds, ctx.compute)
+        dh = mxfp8_matmul_pq(dq, ds, wout_dq, wout_ds, ctx.compute, out_pad=_PITCH_PAD)
         pq, ps, ptq, pts = swiglu_bwd_mx_dual(dh, gu, stage_major=ctx.stage_major)
         # The last three products are independent and none fills the GPU alone (dW has few
         # tiles with a long K): they go down together and share the GPU by work.

@@ -183,13 +183,18 @@ def mxfp8_matmul_pq(
     bq: torch.Tensor,
     b_scale: torch.Tensor,
     out_dtype: torch.dtype = torch.bfloat16,
+    out_pad: int = 0,
 ) -> torch.Tensor:
     """``aq @ bq.T`` from pre-quantized operands, fp32 accumulate.
 
     ``aq (M,K)``, ``bq (N,K)`` e4m3 and ``a_scale (M,K//32)``, ``b_scale (N,K//32)``
     ue8m0 in the natural layout ``quantize_mx`` produces.  Needs only ``K % 32 == 0``.
     A 3-D ``(K // 128, rows, 128)`` code tensor is a stage-major operand (``quantize_mx_dual``).
+    ``out_pad``: the result is a view of an allocation with that many spare elements per row (a row
+    pitch of ``N + out_pad``), for callers that know what pitch suits the kernel reading it next.
     """
+    if out_pad < 0:
+        raise ValueError(f"out_pad={out_pad} must not be negative")
     if aq.dim() == 3 or bq.dim() == 3:
         return mxfp8_matmul_pq_batch([(aq, a_scale, bq, b_scale)], out_dtype)[0]
     if aq.dim() != 2 or bq.dim() != 2 or aq.shape[1] != bq.shape[1]:
@@ -211,7 +216,7 @@ def mxfp8_matmul_pq(
         if t.element_size() != 1:
             raise ValueError(f"codes and scales must be 1-byte tensors, got {t.dtype}")
         tensors.append(t if t.stride(1) == 1 else t.contiguous())
-    out = torch.empty(m, n, device=aq.device, dtype=out_dtype)
+    out = torch.empty(m, n + out_pad, device=aq.device, dtype=out_dtype)[:, :n]
     if m and n:
         _gemm_nt_into(*tensors, out)
     return out
