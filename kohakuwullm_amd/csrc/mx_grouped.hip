@@ -1119,9 +1119,11 @@ struct WgradProblem {
     }
 };
 
-// dW of the experts without rows: zeros.  A plain streaming fill, launched ahead of the GEMM (as
-// part of it, the fills of 58 empty experts cost three times what they cost here).  One block
-// per (expert, 64 rows).
+// dW of the experts without rows: zeros.  A plain streaming fill, launched ahead of the GEMM.  (As
+// part of it, in one burst, the fills of 58 empty experts cost three times what they cost here: vector
+// memory operations retire in order, so the first stage's wait for its copies waits for every store
+// issued before them.  Spread over the K stages, a few stores per thread in front of each stage's
+// copies, they cost the GEMM exactly the 14 us the separate launch takes.)  One block per (expert, 64 rows).
 template <int CDT>
 __global__ __launch_bounds__(256) void wgrad_zero_kernel(WgradArgs p, int chunks) {
     const int e = blockIdx.x / chunks, m0 = (blockIdx.x % chunks) * 64;
