@@ -300,7 +300,21 @@ def _expert_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
 
         dw_out[i] = ora.gemm_nt(*qc(a_out[lo:hi]), *qc(h[lo:hi]))
         dw_in[i] = ora.gemm_nt(*qc(dpre16[lo:hi]), *qc(xg[lo:hi]))
-    return dict(out=out, pre=pre, hq=hq, hs=hs, dx=dx, dgate=dgate, dw_in=dw_in, dw_out=dw_out)
+    # The reference's own expert dW (kernels/mxfp8/grouped.py:152-247 called from moe.py:284-325) multiplies 16-bit
+    # operands: gate * dout[token] rounded to the activation dtype against h rebuilt from the stored pre with PyTorch's
+    # 16-bit operators, and dpre against x[token]; fp32 accumulation.  Restated here in fp64 on those 16-bit operands.
+    act = x.dtype
+    a16 = a_out.to(act).double()
+    pre16 = pre.to(act)
+    h16 = (torch.nn.functional.silu(pre16[:, :hid]) * pre16[:, hid:]).double()
+    dw_out16 = torch.zeros_like(dw_out)
+    dw_in16 = torch.zeros_like(dw_in)
+    for i in range(e):
+        lo, hi = off[i], off[i + 1]
+        dw_out16[i] = a16[lo:hi].T @ h16[lo:hi]
+        dw_in16[i] = dpre16[lo:hi].double().T @ xg[lo:hi].double()
+    return dict(out=out, pre=pre, hq=hq, hs=hs, dx=dx, dgate=dgate, dw_in=dw_in, dw_out=dw_out, dw_in16=dw_in16,
+                dw_out16=dw_out16)
 
 
 def _unfused_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
@@ -389,6 +403,11 @@ def test_fused_experts_fwd_bwd(oracle, counts, top_k, dout_scale):
         if c == 0:
             assert (dw_in[i] == 0).all() and (dw_out[i] == 0).all()
     assert dgate.dtype == gate.dtype and dw_in.dtype == torch.bfloat16
+    # Distance to the reference's 16-bit expert dW: this build quantizes both operands of the product to e4m3 along the
+    # tokens, each cast 2.7e-2 away from its operand in relative Frobenius norm, so the product is sqrt(2) x 2.7e-2 =
+    # 3.8e-2 away in expectation.  Held at 5e-2: the quantization and nothing else.
+    assert oracle.rel_error(dw_out, ref["dw_out16"]) < 5e-2
+    assert oracle.rel_error(dw_in, ref["dw_in16"]) < 5e-2
 
     # structural reference without quantization (autograd in fp32): the gap is the e4m3 error of the chain
     xf, wif, wof, gf = (t.float().requires_grad_(True) for t in (x, w_in, w_out, gate))
