@@ -277,6 +277,22 @@ def test_gemm_split_k_accumulate(oracle):
                     _lib.MX_DTYPE[torch.bfloat16], m, n, k, k, k // 32, k, k // 32, n, 1, None, 0)
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(512, 768, 2048, 128), (300, 200, 640, 8), (256, 256, 128, 3)])
+def test_gemm_output_with_spare_elements_per_row(oracle, m, n, k, pad):
+    """`out_pad`: the product lands in a view of an allocation whose rows are `pad` elements longer (the fused MLP's
+    choice for the projection outputs its SwiGLU quantizers read); same bits as the contiguous result, also on a pitch
+    that rules out 16-byte stores."""
+    aq, as_, bq, bs = _operands(oracle, m, n, k)
+    f8 = torch.float8_e4m3fn
+    dev = [aq.to(DEV).view(f8), as_.to(DEV), bq.to(DEV).view(f8), bs.to(DEV)]
+    plain = _mx().mxfp8_matmul_pq(*dev, torch.bfloat16)
+    padded = _mx().mxfp8_matmul_pq(*dev, torch.bfloat16, out_pad=pad)
+    assert padded.shape == (m, n) and padded.stride() == (n + pad, 1)
+    assert torch.equal(padded, plain)
+    with pytest.raises(ValueError):
+        _mx().mxfp8_matmul_pq(*dev, torch.bfloat16, out_pad=-1)
+
+
 def test_gemm_errors():
     mx = _mx()
     f8 = torch.float8_e4m3fn
