@@ -734,9 +734,41 @@ def run_gemm_variants(dev, iters: int) -> dict:
                 row["rel_error"] = round(_rel_error(first, _dequant(aq, sa) @ _dequant(bq, sb).t()), 6)
             row[name] = {"us_median": round(ts[len(ts) // 2] * 1e3, 1), "tflops_median": round(2.0 * m * n * k / ts[len(ts) // 2] / 1e9, 1),
                          "tflops_best": round(2.0 * m * n * k / ts[0] / 1e9, 1), "equal_to_shipped": bool(torch.equal(c, first))}
+        row["vendor_library"] = _vendor_scaled_mm(ops, first, iters)
         rows.append(row)
         del ops
     return {"shapes": rows}
+
+
+def _vendor_scaled_mm(ops, ours, iters: int) -> dict:
+    """The same product through the vendor's GEMM library as PyTorch reaches it (torch._scaled_mm with one ue8m0 scale per 32
+    of K in the natural (rows, K/32) layout), on the same rotating operands: a yardstick beside the shipped kernel, as the
+    reference keeps its cuBLAS route beside its own kernel.  Nothing in the package calls it; a PyTorch build without the
+    block-scaled form reports the error text instead of a time."""
+    import torch
+
+    e8 = getattr(torch, "float8_e8m0fnu", None)
+    if e8 is None or not hasattr(torch, "_scaled_mm"):
+        return {"error": "this PyTorch has no block-scaled _scaled_mm"}
+    state = {"i": 0}
+    out = {}
+
+    def call():
+        aq, sa, bq, sb = ops[state["i"] % len(ops)]
+        state["i"] += 1
+        out["c"] = torch._scaled_mm(aq, bq.t(), scale_a=sa.view(e8), scale_b=sb.view(e8), out_dtype=torch.bfloat16)
+
+    try:
+        ts = _event_times(call, iters, warm=len(ops))
+        state["i"] = 0
+        call()
+        torch.cuda.synchronize()
+    except Exception as ex:  # noqa: BLE001 - whatever the library or the binding refuses
+        return {"error": f"{type(ex).__name__}: {str(ex)[:200]}"}
+    m, k = ops[0][0].shape
+    n = ops[0][2].shape[0]
+    return {"us_median": round(ts[len(ts) // 2] * 1e3, 1), "tflops_median": round(2.0 * m * n * k / ts[len(ts) // 2] / 1e9, 1),
+            "rel_error_to_shipped": round(_rel_error(out["c"], ours.float()), 6)}
 
 
 def standalone_line(args, dev) -> dict:
@@ -752,7 +784,8 @@ def standalone_line(args, dev) -> dict:
         return {"metric": "MXFP8 GEMM TFLOP/s (mx_gemm_nt alone, cold operands, shipped tiling)", "value": round(val, 1), "unit": "TFLOP/s",
                 "ms_per_step": round(secs * 1e3, 4), "dtype": "e4m3 x e4m3, ue8m0 scales, fp32 accumulate, bf16 out", **common,
                 "config": {"workload": "the six products of BASELINE configs[1] and the 8192^3 of configs[4], each alone; the shipped 256x256 "
-                                       "lockstep kernel of the product library against the three kernels of the variants library", **res},
+                                       "lockstep kernel of the product library against the three kernels of the variants library and, as a yardstick, the "
+                                       "vendor library's block-scaled GEMM as torch._scaled_mm reaches it", **res},
                 "roofline": {"kernel": "gemm_nt_kernel", "bound": "mfma", "achieved": round(val, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(val / MFMA_PEAK_TFLOPS, 4), "traffic": None, "peak_measured": peaks["mfma_tflops"],
                              "frac_of_measured": round(val / peaks["mfma_tflops"], 4)}}
