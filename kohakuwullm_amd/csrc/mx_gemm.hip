@@ -227,11 +227,14 @@ struct DenseProblem {
     }
 };
 
-template <typename S, int CDT, int K512>
+// AHEAD: the A operand is fetched two K stages ahead (persistent_gemm); every tile, K-split piece and K slice of the
+// launch must then have at least two stages.  Instantiated for SCALES_VEC16 only, whose K % 512 == 0 makes every
+// one of them a multiple of four stages.
+template <typename S, int CDT, int K512, bool AHEAD = false>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_kernel(DenseArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     DenseProblem<S, CDT> prob(args, (int)blockIdx.x, (int)gridDim.x);
-    persistent_gemm<S, K512>(prob, smem);
+    persistent_gemm<S, K512, DenseProblem<S, CDT>, AHEAD>(prob, smem);
 }
 
 #ifdef MX_BENCH_VARIANTS
@@ -276,7 +279,7 @@ struct DenseBatchArgs {
     int count;
 };
 
-template <typename S, int CDT, int K512>
+template <typename S, int CDT, int K512, bool AHEAD = false>
 __global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     // workgroups go to the XCDs round-robin: this one runs on XCD blockIdx.x % 8
@@ -285,7 +288,7 @@ __global__ __launch_bounds__(S::NTHR) void gemm_nt_batch_kernel(DenseBatchArgs b
     while (j + 1 < b.count && x >= b.x_lo[j + 1]) j++;
     const int nx = b.x_lo[j + 1] - b.x_lo[j];
     DenseProblem<S, CDT> prob(b.prob[j], (x - b.x_lo[j]) + nx * slot, nx * ((int)gridDim.x >> 3));
-    persistent_gemm<S, K512>(prob, smem);
+    persistent_gemm<S, K512, DenseProblem<S, CDT>, AHEAD>(prob, smem);
 }
 
 // Second half of the even K split: each thread owns what one lane of the GEMM epilogue owns
@@ -442,6 +445,17 @@ static inline int workspace_slots(const void *ws, int64_t bytes) {
 }
 
 // Which scale fetch (SCALES_*) a problem's K and scale pointers allow.
+// Whether the A look-ahead (persistent_gemm) is used: from K = 8192 on.  It wins on long contractions (the three of the
+// feed-forward backward, K = 8192 and 16384, in one launch: 443 -> 422 us on one box, 457 -> 442 us on another) and is
+// level or behind on short ones (K = 1536: 180 -> 180 us and 186 -> 192 us on the same two boxes; K = 4096 with its
+// K-split pieces of 16 stages: 107 -> 109 and 110 -> 113 us), where what it costs per tile -- the next tile's first A
+// rows are waited for a stage early, behind a wait the compiler puts in front of the next tile's scale bytes -- is
+// spread over a dozen stages only.
+#ifndef MX_AHEAD_MIN_K
+#define MX_AHEAD_MIN_K 8192
+#endif
+static bool ahead_pays(int64_t K) { return K >= MX_AHEAD_MIN_K; }
+
 static int scale_mode(const DenseArgs &a) {
     if (a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0) return SCALES_VEC16;
     if (a.K % 128 == 0 && aligned(a.as, 4) && aligned(a.bs, 4) && a.ldas % 4 == 0 && a.ldbs % 4 == 0) return SCALES_DWORD;
@@ -494,7 +508,9 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
                                     : launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
     else
 #endif
-        rc = mode == SCALES_VEC16   ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
+        rc = mode == SCALES_VEC16 && ahead_pays(a.K)
+                 ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16, true>>(grid, block, S::LDS_BYTES_AHEAD, st, a)
+             : mode == SCALES_VEC16 ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
              : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
                                     : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
     if (rc != MX_OK) return rc;
@@ -678,7 +694,10 @@ static int batch_dispatch(DenseArgs *probs, int count, float *ws, int ws_slots, 
     }
     b.count = count;
     const dim3 grid((unsigned)cus), block(S::NTHR);
-    const int rc = mode == SCALES_VEC16 ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, b)
+    bool ahead = mode == SCALES_VEC16;
+    for (int j = 0; j < count; j++) ahead = ahead && ahead_pays(probs[j].K);
+    const int rc = ahead ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_VEC16, true>>(grid, block, S::LDS_BYTES_AHEAD, st, b)
+                   : mode == SCALES_VEC16 ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, b)
                    : mode == SCALES_DWORD
                        ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, b)
                        : launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, b);

@@ -95,6 +95,35 @@ __device__ __forceinline__ uint32_t lds_addr(const void *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }
 
+// A workgroup-wide event counter in LDS for the look-ahead of the A operand (see persistent_gemm): lane 0 of a wave adds
+// one once the wave's A fragments of a stage are in registers; a wave about to overwrite that stage's A rows waits until
+// all waves have.  Both are single asm statements -- no control flow the compiler can see, so the stage body stays one
+// basic block -- and both wait on lgkmcnt(0) first: LDS operations return in order.
+__device__ __forceinline__ void lds_count_up(uint32_t counter) {
+    uint64_t saved;
+    uint32_t one = 1;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\t"
+                 "s_mov_b64 %0, exec\n\t"
+                 "s_mov_b64 exec, 1\n\t"
+                 "ds_add_u32 %1, %2\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "v"(counter), "v"(one)
+                 : "memory");
+}
+__device__ __forceinline__ void lds_count_wait(uint32_t counter, uint32_t target) {
+    uint32_t v, sv;
+    asm volatile("lds_count_wait_%=:\n\t"
+                 "ds_read_b32 %0, %2\n\t"
+                 "s_waitcnt lgkmcnt(0)\n\t"
+                 "v_readfirstlane_b32 %1, %0\n\t"
+                 "s_cmp_lt_u32 %1, %3\n\t"
+                 "s_cbranch_scc1 lds_count_wait_%="
+                 : "=&v"(v), "=&s"(sv)
+                 : "v"(counter), "s"(target)
+                 : "memory", "scc");
+}
+
 __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     uint64_t u = (uint64_t)p;
     uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
@@ -117,6 +146,7 @@ struct GemmShape {
     static constexpr int PA = BM + 16, PB = BN + 16;
     static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
     static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B);
+    static constexpr int LDS_BYTES_AHEAD = LDS_BYTES + 64;  // + the event counter of the A look-ahead
     static constexpr bool TWO_ROWS = BM + BN > NTHR;
     static_assert(NT == 8 || NT == 4, "a lane's NT sub-tiles are NT consecutive N: one 16-byte (or 8-byte) store");
     static_assert(WTM % 16 == 0, "a wave's M extent must be a multiple of 16");
@@ -265,6 +295,14 @@ __device__ __forceinline__ void issue_stage(const IssueCtx<S> &c, const Lane &L,
     static_for<CopyRuns<S>::N>([&](auto r) { CopyRuns<S>::template issue<r.value>(c, L, kt, ga, gb, la, lb); });
 }
 
+// The A rows of stage `kt` alone (the look-ahead's second stage in a kernel's prologue).
+template <typename S>
+__device__ __forceinline__ void issue_a(const IssueCtx<S> &c, const Lane &L, int kt, uint8_t *ldsA, int buf) {
+    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt * c.a_ks - COPY_BIAS);
+    const uint32_t la = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf * S::DATA_A + L.wave * S::QA * 1024);
+    static_for<CopyRuns<S>::RA>([&](auto r) { CopyRuns<S>::template issue<r.value>(c, L, kt, ga, ga, la, la); });
+}
+
 // How a row's scale bytes are fetched: one 16-byte load per 512 of K (K % 512 == 0, 16-byte
 // aligned rows), one dword per stage (K % 128 == 0, 4-byte aligned rows), or byte by byte (any
 // K % 32 == 0 and any pitch; blocks past the end of K read as scale byte 0).  SCALES_QUAD: one
@@ -325,15 +363,22 @@ __device__ __forceinline__ void park_scales(int srow, uint32_t *ldsSA, uint32_t 
 // 64 bytes per clock, so the 64 KB a stage needs occupy it for ~1000 clocks per CU; issued in
 // one burst at the top of the stage they stall every wave (and the MFMA pipe) for that long,
 // issued late they would not land before the stage-ending barrier.
-template <typename S, int OPSEL>
+//
+// AHEAD (the A look-ahead, see persistent_gemm): the stage fetches the B rows of stage `kt_next` into buffer `buf_next`
+// in its first steps and, in steps 4 and 5, the A rows of stage `kt_a` of the tile `ca` describes -- the stage after
+// `kt_next` in the workgroup's sequence of stages -- into the A half of the buffer it is itself reading, once every wave
+// has its A fragments of this stage in registers (`counter` has reached `target`).
+template <typename S, int OPSEL, bool AHEAD = false>
 __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, const uint8_t *__restrict__ lb, int a_lo,
                                               int a_hi, int b_lo, int b_hi, const int (&sa)[S::MT],
                                               const int (&sb)[S::NT], v4f (&acc)[S::MT][S::NT],
                                               const IssueCtx<S> &c, const Lane &L, int kt_next, uint8_t *ldsA,
-                                              uint8_t *ldsB, int buf_next) {
-    const uint8_t *ga = uniform_ptr(c.a_base + (int64_t)kt_next * c.a_ks - COPY_BIAS);
+                                              uint8_t *ldsB, int buf_next, const IssueCtx<S> &ca, int kt_a,
+                                              uint32_t counter, uint32_t target) {
+    const uint8_t *ga = uniform_ptr((AHEAD ? ca.a_base + (int64_t)kt_a * ca.a_ks : c.a_base + (int64_t)kt_next * c.a_ks) - COPY_BIAS);
     const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt_next * c.b_ks - COPY_BIAS);
-    const uint32_t wa = __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + buf_next * S::DATA_A + L.wave * S::QA * 1024);
+    const uint32_t wa =
+        __builtin_amdgcn_readfirstlane(lds_addr(ldsA) + (AHEAD ? buf_next ^ 1 : buf_next) * S::DATA_A + L.wave * S::QA * 1024);
     const uint32_t wb = __builtin_amdgcn_readfirstlane(lds_addr(ldsB) + buf_next * S::DATA_B + L.wave * S::QB * 1024);
     typedef CopyRuns<S> Runs;
 
@@ -356,9 +401,13 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
         v4i hi = *(const v4i *)(la + a_hi + i * (16 * 128));
         afr[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
+    if (AHEAD) lds_count_up(counter);  // this wave's A fragments are in registers
     __builtin_amdgcn_sched_barrier(0);
+    constexpr int A_STEP = S::NT / 2;  // AHEAD: the A runs go out in steps A_STEP, A_STEP + 1, ..., the B runs in steps 0, 1, ...
+    static_assert(!AHEAD || (Runs::RA <= S::NT - A_STEP && Runs::RB <= A_STEP), "the runs of a stage fit its two halves");
     static_for<S::NT>([&](auto jc) {
         constexpr int j = jc.value;
+        if constexpr (AHEAD && j == A_STEP) lds_count_wait(counter, target);
         if (j + 1 < S::NT) {
             v4i lo = *(const v4i *)(lb + b_lo + (j + 1) * (16 * 128));
             v4i hi = *(const v4i *)(lb + b_hi + (j + 1) * (16 * 128));
@@ -366,8 +415,13 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
         }
         // run r goes out in step r STEPS / N: evenly over the first half of the stage
         static_for<Runs::N>([&](auto r) {
-            if constexpr (r.value * STEPS / Runs::N == j && j < STEPS)
+            if constexpr (AHEAD) {
+                constexpr bool isb = r.value >= Runs::RA;
+                if constexpr (isb && r.value - Runs::RA == j) Runs::template issue<r.value>(c, L, kt_next, ga, gb, wa, wb);
+                if constexpr (!isb && A_STEP + r.value == j) Runs::template issue<r.value>(ca, L, kt_a, ga, gb, wa, wb);
+            } else if constexpr (r.value * STEPS / Runs::N == j && j < STEPS) {
                 Runs::template issue<r.value>(c, L, kt_next, ga, gb, wa, wb);
+            }
         });
 #pragma unroll
         for (int i = 0; i < S::MT; i++)
@@ -412,8 +466,22 @@ struct LdsScratch {
 //                                           constant P::NST for the whole wave, else -1
 //   int  P::kb_end                          scale bytes per row (bound for predicated fetches)
 //   bool P::EARLY_WAIT                      wait for the next tile's first stage before the epilogue (see the tile loop)
-template <typename S, int K512, typename P>  // K512: one of SCALES_*
+//
+// AHEAD, the A look-ahead.  A stage's copies are all waited for at the end of the stage that issues them, because the
+// stage after it reads them; the wait is for the slowest of 64 copies per CU, and a vector-memory wait is for everything
+// older, so nothing may be left in flight across the barrier.  The A rows of a stage, however, are dead a few hundred
+// clocks into it (every wave reads its A fragments first and holds them), while its B rows are read to the end.  With
+// AHEAD the workgroup therefore fetches A TWO stages ahead -- stage g, in its second half, fetches the A rows of stage
+// g + 2 into the A half of its own buffer, once an event counter in LDS says that all eight waves have their A fragments
+// -- and B one stage ahead as before.  The stage-ending wait then leaves the wave's youngest S::QA copies, those A rows,
+// in flight: they have another whole stage to land.  Stages are numbered through the workgroup's whole sequence of
+// tiles, so the last two stages of a tile fetch the A rows of the next tile's first two; every tile must therefore have
+// at least two stages (the caller's guarantee), and the epilogue may not use the stage buffer as scratch (no EARLY_WAIT
+// policy does both).  Same products bit for bit: the MFMA sequence does not change.  Measured inside the feed-forward
+// step: the batched launch of the three long contractions 457 -> 429 us, the K = 1536 products 1 % faster.
+template <typename S, int K512, typename P, bool AHEAD = false>  // K512: one of SCALES_*
 __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
+    static_assert(!(AHEAD && P::EARLY_WAIT), "an epilogue that borrows the stage buffer cannot share it with the look-ahead");
     uint8_t *const ldsA = smem;                                                  // [2][BM*128]
     uint8_t *const ldsB = smem + 2 * S::DATA_A;                                  // [2][BN*128]
     uint32_t *const ldsSA = (uint32_t *)(smem + 2 * (S::DATA_A + S::DATA_B));    // [2][4][PA]
@@ -429,11 +497,14 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     const int a_rd = a_row * 128 + ((L.g ^ swz_a(a_row)) << 4);
     const int b_rd = b_row * 128 + ((L.g ^ swz_a(b_row)) << 4);
 
+    const uint32_t counter = lds_addr(smem + S::LDS_BYTES);  // AHEAD only: waves whose A fragments are in registers, over all stages
     typename P::Tile cur, nxt;
     if (!prob.next(cur)) return;
     bool has_next = prob.next(nxt);
-    IssueCtx<S> ctx;
+    IssueCtx<S> ctx;   // the tile whose B rows and scale bytes are being fetched
+    IssueCtx<S> ctxa;  // AHEAD: the tile whose A rows are being fetched (the next tile's, from a tile's second-to-last stage on)
     prob.context(cur, L, ctx);
+    if (AHEAD) ctxa = ctx;
 
     int gstage = 0;  // stages issued so far, over all tiles: LDS data buffer = gstage & 1
     int gsuper = 0;  // super-steps so far: LDS scale buffer = gsuper & 1
@@ -444,6 +515,10 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);
         if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);
         issue_stage<S>(ctx, L, ctx.kt0, ldsA, ldsB, 0);
+        if (AHEAD) {
+            issue_a<S>(ctx, L, ctx.kt0 + 1, ldsA, 1);
+            if (L.tid == 0) *(volatile uint32_t *)(smem + S::LDS_BYTES) = 0;
+        }
         if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
         if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
     }
@@ -498,10 +573,22 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             } else {                                                                                          \
                 kt_issue = kt0 + k; /* nothing left to fetch: a harmless re-read of this stage */             \
             }                                                                                                 \
-            compute_stage<S, SIDX>(ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64, b_rd,     \
-                                   b_rd ^ 64, sa, sb, acc, ctx, L, kt_issue, ldsA, ldsB, buf ^ 1);            \
+            /* AHEAD: the A rows two stages on: this tile's, or the next tile's first two (its context  */    \
+            /* from the second-to-last stage on), or, with no tile left, a re-read nobody will look at. */    \
+            int kt_a = kt0 + k + 2;                                                                           \
+            if (AHEAD && k + 2 >= KT) {                                                                       \
+                if (has_next) {                                                                               \
+                    if (k + 2 == KT) prob.context(nxt, L, ctxa);                                              \
+                    kt_a = ctxa.kt0 + (k + 2 - KT);                                                           \
+                } else {                                                                                      \
+                    kt_a = kt0 + k;                                                                           \
+                }                                                                                             \
+            }                                                                                                 \
+            compute_stage<S, SIDX, AHEAD>(ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64,    \
+                                          b_rd, b_rd ^ 64, sa, sb, acc, ctx, L, kt_issue, ldsA, ldsB,         \
+                                          buf ^ 1, ctxa, kt_a, counter, (uint32_t)(gstage + 1) * S::NW);      \
             if (!last) {                                                                                      \
-                wait_vm_allow_c<0>();                                                                         \
+                wait_vm_allow_c<AHEAD ? S::QA : 0>();                                                         \
                 __syncthreads();                                                                              \
             }                                                                                                 \
             gstage++;                                                                                         \

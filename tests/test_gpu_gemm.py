@@ -152,6 +152,8 @@ SPLIT_SHAPES = [
     (2048, 1536, 2048),  # 48 tiles
     (4352, 4096, 1024),  # one whole round of 256 tiles, then 16 more that are split
     (768, 512, 8160),  # K % 128 == 96: the partial stage ends the last piece of every tile
+    (700, 500, 8704),  # ragged edges under the A look-ahead (K >= 8192, K % 512 == 0): 68 stages in pieces, tiles of both kinds per workgroup
+    (2304, 2560, 8192),  # 90 whole tiles under the look-ahead, none split
 ]
 
 
@@ -173,6 +175,7 @@ def test_gemm_even_k_split(oracle, m, n, k):
 
 BATCHES = [
     [(512, 384, 1024), (384, 256, 4096), (256, 256, 8192)],  # the shape mix of a backward: short K many tiles, long K few
+    [(512, 384, 8192), (300, 256, 16384), (256, 700, 8704)],  # every K >= 8192: the batched launch under the A look-ahead, K slices included
     [(300, 200, 640), (64, 64, 96)],  # ragged, and one problem only the generic kernel takes: run in turn
     [(256, 512, 512)],
     [(256, 256, 256)] * 6,  # more than one launch's worth
