@@ -137,6 +137,10 @@ struct DenseProblem {
         }
         c.srow0 = scale_row(t, L.tid < S::BM + S::BN ? L.tid : 0);
         c.srow1 = S::TWO_ROWS ? scale_row(t, L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
+        // SCALES_COPY: the same row as srow0, as an offset into its scale matrix (the launcher checked that it fits)
+        c.sa_base = p.as;
+        c.sb_base = p.bs;
+        c.s_voff = (uint32_t)(c.srow0 - (L.tid < S::BM ? p.as : p.bs));
     }
 
 #ifdef MX_BENCH_VARIANTS
@@ -445,16 +449,20 @@ static inline int workspace_slots(const void *ws, int64_t bytes) {
 }
 
 // Which scale fetch (SCALES_*) a problem's K and scale pointers allow.
-// Whether the A look-ahead (persistent_gemm) is used: from K = 8192 on.  It wins on long contractions (the three of the
-// feed-forward backward, K = 8192 and 16384, in one launch: 443 -> 422 us on one box, 457 -> 442 us on another) and is
-// level or behind on short ones (K = 1536: 180 -> 180 us and 186 -> 192 us on the same two boxes; K = 4096 with its
-// K-split pieces of 16 stages: 107 -> 109 and 110 -> 113 us), where what it costs per tile -- the next tile's first A
-// rows are waited for a stage early, behind a wait the compiler puts in front of the next tile's scale bytes -- is
-// spread over a dozen stages only.
+// Whether the A look-ahead (persistent_gemm) is used: whenever the scale bytes can go through the copy engine
+// (SCALES_COPY) and K spans at least two groups of four stages.  It wins on long contractions (the three of the
+// feed-forward backward, K = 8192 and 16384, in one launch: 442 -> 416 us) and is level on short ones (K = 1536:
+// 183 -> 183 us; K = 4096 with its K-split pieces of 16 stages: 105 -> 107 us).  (With the scale bytes loaded through
+// registers it lost 3 % on the short ones: the compiler, which cannot see the copies, put a full vector-memory wait in
+// front of every use of those loads, once per four stages and once per tile, and the A rows meant to stay in flight
+// were waited for half a stage after their issue.)
 #ifndef MX_AHEAD_MIN_K
-#define MX_AHEAD_MIN_K 8192
+#define MX_AHEAD_MIN_K 1024
 #endif
-static bool ahead_pays(int64_t K) { return K >= MX_AHEAD_MIN_K; }
+static bool ahead_pays(const DenseArgs &a) {
+    // its scale bytes go through the copy engine, whose lane offsets are 32 bits
+    return a.K >= MX_AHEAD_MIN_K && (int64_t)a.M * a.ldas < ((int64_t)1 << 32) && (int64_t)a.N * a.ldbs < ((int64_t)1 << 32);
+}
 
 static int scale_mode(const DenseArgs &a) {
     if (a.K % 512 == 0 && aligned(a.as, 16) && aligned(a.bs, 16) && a.ldas % 16 == 0 && a.ldbs % 16 == 0) return SCALES_VEC16;
@@ -508,8 +516,8 @@ static int launch_tiled(DenseArgs a, float *ws, int ws_slots, hipStream_t st, bo
                                     : launch_with_lds<gemm_nt_phased_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
     else
 #endif
-        rc = mode == SCALES_VEC16 && ahead_pays(a.K)
-                 ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16, true>>(grid, block, S::LDS_BYTES_AHEAD, st, a)
+        rc = mode == SCALES_VEC16 && ahead_pays(a)
+                 ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_COPY, true>>(grid, block, S::LDS_BYTES_AHEAD, st, a)
              : mode == SCALES_VEC16 ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, a)
              : mode == SCALES_DWORD ? launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a)
                                     : launch_with_lds<gemm_nt_kernel<S, CDT, SCALES_BYTES>>(grid, block, S::LDS_BYTES, st, a);
@@ -695,8 +703,8 @@ static int batch_dispatch(DenseArgs *probs, int count, float *ws, int ws_slots, 
     b.count = count;
     const dim3 grid((unsigned)cus), block(S::NTHR);
     bool ahead = mode == SCALES_VEC16;
-    for (int j = 0; j < count; j++) ahead = ahead && ahead_pays(probs[j].K);
-    const int rc = ahead ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_VEC16, true>>(grid, block, S::LDS_BYTES_AHEAD, st, b)
+    for (int j = 0; j < count; j++) ahead = ahead && ahead_pays(probs[j]);
+    const int rc = ahead ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_COPY, true>>(grid, block, S::LDS_BYTES_AHEAD, st, b)
                    : mode == SCALES_VEC16 ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_VEC16>>(grid, block, S::LDS_BYTES, st, b)
                    : mode == SCALES_DWORD
                        ? launch_with_lds<gemm_nt_batch_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, b)

@@ -146,7 +146,8 @@ struct GemmShape {
     static constexpr int PA = BM + 16, PB = BN + 16;
     static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
     static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B);
-    static constexpr int LDS_BYTES_AHEAD = LDS_BYTES + 64;  // + the event counter of the A look-ahead
+    // + the staging area of SCALES_COPY (16 bytes per row of A and B) and the event counter of the A look-ahead
+    static constexpr int LDS_BYTES_AHEAD = LDS_BYTES + 16 * (BM + BN) + 64;
     static constexpr bool TWO_ROWS = BM + BN > NTHR;
     static_assert(NT == 8 || NT == 4, "a lane's NT sub-tiles are NT consecutive N: one 16-byte (or 8-byte) store");
     static_assert(WTM % 16 == 0, "a wave's M extent must be a multiple of 16");
@@ -206,6 +207,9 @@ struct IssueCtx {
     // per copy q: byte offset of this lane's chunk from the base, plus copy_bias(q) (see dma16_run2)
     uint32_t a_voff[S::QA], b_voff[S::QB];
     const uint8_t *srow0, *srow1;  // scale rows tid and tid + NTHR of the [A rows; B rows] list
+    // SCALES_COPY: the scale matrices and this lane's byte offset to the start of scale row tid of the list
+    const uint8_t *sa_base, *sb_base;
+    uint32_t s_voff;
     int kt0, kt1;                  // K range in 128-byte stages (absolute)
     // K % 128 != 0: stage tail_kt holds only tail_bytes of K.  Its copies re-read the stage's first
     // chunk in place of chunks past the end of the row (never past the matrix), and those
@@ -311,7 +315,14 @@ __device__ __forceinline__ void issue_a(const IssueCtx<S> &c, const Lane &L, int
 // caller guarantees to lie inside the row's pitch.  Against SCALES_DWORD it asks the L2 for a
 // row's line once per four stages instead of once per stage: 512 rows x 4 bytes a stage is half
 // as many lines again as the stage's codes.
-enum { SCALES_VEC16 = 0, SCALES_DWORD = 1, SCALES_BYTES = 2, SCALES_QUAD = 3 };
+// SCALES_COPY: the rows' 16 scale bytes per 512 of K go from memory to LDS through the copy engine, like the codes (one
+// copy per wave and four stages, into a staging area of 16 bytes per row), and the thread that would have loaded a row
+// takes it from there when it transposes it into the planes.  No registers hold scale bytes in flight, and -- what it
+// is for -- the K loop holds no vector load the compiler can see: in front of such a load's use it puts a full
+// vector-memory wait, which under the A look-ahead waits for copies that are meant to stay in flight.  A row is staged
+// and transposed by the same wave, so the wave's own vector-memory waits order the two.  Needs what SCALES_VEC16 needs
+// and scale matrices under 4 GB; a policy fills IssueCtx::s_voff / sa_base / sb_base for it.
+enum { SCALES_VEC16 = 0, SCALES_DWORD = 1, SCALES_BYTES = 2, SCALES_QUAD = 3, SCALES_COPY = 4 };
 
 // 16 scale bytes (4 stages x 4 blocks) of one row starting at scale column kb0.
 template <int MODE>
@@ -353,6 +364,24 @@ __device__ __forceinline__ void park_scales(int srow, uint32_t *ldsSA, uint32_t 
 #pragma unroll
         for (int gg = 0; gg < 4; gg++) dst[gg * S::PB] = t[gg];
     }
+}
+
+// SCALES_COPY: the 16 scale bytes from scale column kb0 of this workgroup's BM + BN rows into scale buffer `sbuf`
+// (row r of the list at byte 16 r): one copy per wave, waves 0 .. BM / 64 - 1 the A rows.
+template <typename S>
+__device__ __forceinline__ void issue_scales(const IssueCtx<S> &c, const Lane &L, int kb0, uint8_t *raw) {
+    static_assert(S::BM % 64 == 0 && S::BM + S::BN == S::NTHR, "one row of the list per thread, whole waves of A rows");
+    const uint8_t *base = uniform_ptr((L.wave < S::BM / 64 ? c.sa_base : c.sb_base) + kb0);
+    const uint32_t lds = __builtin_amdgcn_readfirstlane(lds_addr(raw) + L.wave * 1024);
+    dma16(base, c.s_voff, lds);
+}
+// ... and from the staging area into scale buffer `sbuf` of the planes (the thread's own row; the copy has landed).
+template <typename S>
+__device__ __forceinline__ void park_staged(const Lane &L, const uint8_t *raw, uint32_t *ldsSA, uint32_t *ldsSB, int sbuf) {
+    asm volatile("" ::: "memory");  // behind the vector-memory wait that covers the copy
+    const v4i t = *(const v4i *)(raw + L.tid * 16);
+    const uint32_t d[4] = {(uint32_t)t[0], (uint32_t)t[1], (uint32_t)t[2], (uint32_t)t[3]};
+    park_scales<S>(L.tid, ldsSA, ldsSB, sbuf, d);
 }
 
 // One K stage of the workgroup tile: this wave's MT x NT accumulators advance by 128 of K,
@@ -487,6 +516,9 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     uint32_t *const ldsSA = (uint32_t *)(smem + 2 * (S::DATA_A + S::DATA_B));    // [2][4][PA]
     uint32_t *const ldsSB = ldsSA + 2 * 4 * S::PA;                               // [2][4][PB]
 
+    constexpr bool COPY = K512 == SCALES_COPY;
+    uint8_t *const rawS = smem + S::LDS_BYTES;  // SCALES_COPY: the staging area, [BM + BN rows][16 bytes]
+
     const Lane L = lane_of<S>();
     const bool has_row0 = L.tid < S::BM + S::BN;
     const int kb_end = prob.kb_end;
@@ -497,7 +529,8 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     const int a_rd = a_row * 128 + ((L.g ^ swz_a(a_row)) << 4);
     const int b_rd = b_row * 128 + ((L.g ^ swz_a(b_row)) << 4);
 
-    const uint32_t counter = lds_addr(smem + S::LDS_BYTES);  // AHEAD only: waves whose A fragments are in registers, over all stages
+    // AHEAD only: waves whose A fragments are in registers, over all stages
+    const uint32_t counter = lds_addr(smem + S::LDS_BYTES + 16 * (S::BM + S::BN));
     typename P::Tile cur, nxt;
     if (!prob.next(cur)) return;
     bool has_next = prob.next(nxt);
@@ -512,17 +545,24 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     // prologue of the first tile
     {
         uint32_t d0[4], d1[4];
-        if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);
-        if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);
+        if constexpr (COPY) {
+            issue_scales<S>(ctx, L, ctx.kt0 * 4, rawS);
+        } else {
+            if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);
+            if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);
+        }
         issue_stage<S>(ctx, L, ctx.kt0, ldsA, ldsB, 0);
         if (AHEAD) {
             issue_a<S>(ctx, L, ctx.kt0 + 1, ldsA, 1);
-            if (L.tid == 0) *(volatile uint32_t *)(smem + S::LDS_BYTES) = 0;
+            if (L.tid == 0) *(volatile uint32_t *)(smem + S::LDS_BYTES + 16 * (S::BM + S::BN)) = 0;
         }
-        if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
-        if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
+        if constexpr (!COPY) {
+            if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, 0, d0);
+            if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, 0, d1);
+        }
     }
     wait_vm_allow_c<0>();
+    if constexpr (COPY) park_staged<S>(L, rawS, ldsSA, ldsSB, 0);
     __syncthreads();
 
     v4f acc[S::MT][S::NT];
@@ -558,17 +598,29 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             int kt_issue = kt0 + k + 1;                                                                       \
             if (!last) {                                                                                      \
                 if (SIDX == 3) {                                                                              \
-                    if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, sbuf ^ 1, d0);                          \
-                    if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, sbuf ^ 1, d1);             \
+                    if constexpr (COPY) {                                                                     \
+                        park_staged<S>(L, rawS, ldsSA, ldsSB, sbuf ^ 1);                                      \
+                    } else {                                                                                  \
+                        if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, sbuf ^ 1, d0);                      \
+                        if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, sbuf ^ 1, d1);         \
+                    }                                                                                         \
                 }                                                                                             \
                 if (SIDX == 0 && ss + 1 < nsuper) {                                                           \
-                    if (has_row0) load_scales<K512>(ctx.srow0, (kt0 + (ss + 1) * 4) * 4, kb_end, d0);         \
-                    if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, (kt0 + (ss + 1) * 4) * 4, kb_end, d1);      \
+                    if constexpr (COPY) {                                                                     \
+                        issue_scales<S>(ctx, L, (kt0 + (ss + 1) * 4) * 4, rawS);                              \
+                    } else {                                                                                  \
+                        if (has_row0) load_scales<K512>(ctx.srow0, (kt0 + (ss + 1) * 4) * 4, kb_end, d0);     \
+                        if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, (kt0 + (ss + 1) * 4) * 4, kb_end, d1);  \
+                    }                                                                                         \
                 }                                                                                             \
             } else if (has_next) {                                                                            \
                 prob.context(nxt, L, ctx);                                                                    \
-                if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);                          \
-                if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);                       \
+                if constexpr (COPY) {                                                                         \
+                    issue_scales<S>(ctx, L, ctx.kt0 * 4, rawS);                                               \
+                } else {                                                                                      \
+                    if (has_row0) load_scales<K512>(ctx.srow0, ctx.kt0 * 4, kb_end, d0);                      \
+                    if (S::TWO_ROWS) load_scales<K512>(ctx.srow1, ctx.kt0 * 4, kb_end, d1);                   \
+                }                                                                                             \
                 kt_issue = ctx.kt0;                                                                           \
             } else {                                                                                          \
                 kt_issue = kt0 + k; /* nothing left to fetch: a harmless re-read of this stage */             \
@@ -612,6 +664,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         // scales are parked then (their planes were last read two super-steps ago, with a barrier
         // since), and the barrier behind the epilogue publishes both.  The epilogue's own stores then
         // need no wait at all and drain under the next tile's K loop instead of in front of it.
+        static_assert(!(COPY && P::EARLY_WAIT), "the fused epilogues borrow a scale plane and keep the planes");
         if (P::EARLY_WAIT && has_next) {
             wait_vm_allow_c<0>();
             if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
@@ -619,7 +672,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         }
         const int stores = prob.epilogue(cur, L, acc, LdsScratch{ldsA + lastbuf * S::DATA_A, ldsB + lastbuf * S::DATA_B,
                                             (uint8_t *)(ldsSA + ((gsuper - 1) & 1) * 4 * S::PA)});
-        if (!P::EARLY_WAIT && has_next) {
+        if (!P::EARLY_WAIT && has_next && !COPY) {
             if (has_row0) park_scales<S>(L.tid, ldsSA, ldsSB, gsuper & 1, d0);
             if (S::TWO_ROWS) park_scales<S>(L.tid + S::NTHR, ldsSA, ldsSB, gsuper & 1, d1);
         }
@@ -628,6 +681,7 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             if (stores == P::NST) wait_vm_allow_c<P::NST>();
             else wait_vm_allow_c<0>();
         }
+        if constexpr (COPY) park_staged<S>(L, rawS, ldsSA, ldsSB, gsuper & 1);  // the next tile's first scale bytes: staged in the last stage
         __syncthreads();
         cur = nxt;
         has_next = prob.next(nxt);
