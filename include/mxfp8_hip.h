@@ -304,6 +304,8 @@ int mx_grouped_gemm_nt(const uint8_t *xq, const uint8_t *xs, int64_t a_rows, int
  * also quantized along the tokens, into the padded layout of mx_quantize_cols_grouped
  * ((H,Mpad), (H,Mpad/32); with E == 1 and M % 128 == 0 that is plain (H,M)): the operand of
  * GEMM2's WGRAD, bit-identical to mx_quantize_cols_grouped(pre, source = SwiGLU).
+ * ldhtq == 128 with more than one 128-position tile in the padded space selects the stage-major
+ * form of htq described at mx_quantize_cols_grouped: (Mpad/128, H, 128).
  * With E == 1 this is the dense SwiGLU block's first projection with the activation and both
  * casts in the epilogue (GLUMLP.forward, src/kohakuwullm/models/components/mlp.py:68-73).
  * Replaces _experts_gemm1 / launch_gemm1 (src/kohakuwullm/kernels/mxfp8/experts.py:25-135,225-275).
@@ -354,6 +356,7 @@ int mx_experts_combine(const void *y, int64_t ldy, const int32_t *order, const i
  * Optional (both or neither): ptq (2H,Mpad), pts (2H,Mpad/32) receive the stored (rounded)
  * dpre quantized along the tokens in the padded layout of mx_quantize_cols_grouped, bit for
  * bit what that quantizer makes of dpre; dpre itself may then be NULL and is not written.
+ * ldptq == 128 selects the stage-major form of ptq, (Mpad/128, 2H, 128), as there.
  * Replaces _experts_gemm2_dgrad (src/kohakuwullm/kernels/mxfp8/experts_bwd.py:29-164); with
  * ptq it also stands in for the pass over the stored dpre that feeds GEMM1's WGRAD
  * (_launch_wgrad(dpre, x, ...), src/kohakuwullm/kernels/mxfp8/moe.py:311-324).
@@ -377,6 +380,10 @@ int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int64_t T, int6
  *           grouped_mxfp8_wgrad_kernel (src/kohakuwullm/kernels/mxfp8/grouped.py:152-247);
  * source 1: silu(x[m][c]) * x[m][C + c] from the stored pre-activation (M,2C) -- the h the
  *           reference rebuilds in src/kohakuwullm/kernels/mxfp8/moe.py:288-290.
+ * Stage-major codes: ldqT == 128 (with Mpad > 128, always the case for M > 0) stores qT as
+ * (Mpad/128, C, 128) -- byte (c, pos) at (pos/128) * C * 128 + c * 128 + pos % 128 -- so that a K stage
+ * of a WGRAD tile is one contiguous run; the same bytes, sT unchanged.  mx_grouped_wgrad_nt takes
+ * either form per operand.
  */
 int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, int64_t C, int source,
                              const int32_t *index, const void *row_scale, int row_scale_dtype,
@@ -389,6 +396,8 @@ int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, int64_t C, i
  * (stride_dwe, lddw) in elements.  An expert without rows gets zeros.  The MXFP8 form of
  * grouped_mxfp8_wgrad_kernel / _launch_wgrad (grouped.py:152-247, moe.py:64-99), which
  * multiply in 16 bits.
+ * lda == 128 / ldb == 128: that operand's codes are stage-major, (Mpad/128, N, 128) / (Mpad/128, Kout, 128),
+ * as mx_quantize_cols_grouped, mx_experts_gemm1 and mx_experts_gemm2_dgrad write them on request.
  * When both scale pitches leave 12 readable bytes behind a row's last stage (ldas, ldbs >=
  * mpad/32 + 12) the kernel fetches a row's scale bytes 16 at a time instead of 4.
  * workspace as in mx_gemm_nt: with mx_gemm_workspace_bytes() of it the K stages of the experts that

@@ -46,6 +46,7 @@ struct GroupedArgs {
     int64_t ldhq, ldhs;
     uint8_t *htq, *hts;  // GEMM1 out (optional): h quantized along the tokens, (H,Mpad), (H,Mpad/32)
     int64_t ldhtq, ldhts;
+    int64_t htq_ks;  // 0, or htq stage-major: the 128 positions of panel j of every row together, panel j at j * htq_ks, row r at r * 128
     void *pre;  // GEMM1 out (optional) / DGRAD2 in: (M,2H) 16-bit
     int64_t ldpre;
     void *dpre;  // DGRAD2 out: (M,2H) 16-bit
@@ -381,6 +382,13 @@ struct GroupedProblem {
         return interior ? NST : -1;
     }
 
+    // Byte offset in the token-axis code matrix of 16-byte chunk `ch` of a tile's positions (the tile starts at padded
+    // position `pbase`, a multiple of 128) in row `row`: row-major, or stage-major panels of 128 positions.
+    __device__ __forceinline__ int64_t token_axis_offset(int row, int64_t pbase, int ch) const {
+        return p.htq_ks ? ((pbase >> 7) + (ch >> 3)) * p.htq_ks + (int64_t)row * 128 + (ch & 7) * 16
+                        : (int64_t)row * p.ldhtq + pbase + ch * 16;
+    }
+
     // ---- GEMM1: sub-tiles 0-3 are gate, 4-7 value of the lane's 4 hidden units
     // Outputs: pre (rounded accumulators), h quantized along the hidden axis (hq, hs) for GEMM2,
     // and, when htq is given, h quantized along the tokens for GEMM2's WGRAD.  The token-axis
@@ -479,7 +487,7 @@ struct GroupedProblem {
             const bool part_ok = t.row0 + (ch >> 3) * 128 < t.end;
             if (t.n0 + col < p.N && part_ok) {
                 const v4i w = *(const v4i *)(lds.a + col * S::BM + (((ch ^ (col >> 2)) & (CH - 1)) << 4));
-                *(v4i *)(p.htq + (int64_t)(t.n0 + col) * p.ldhtq + pbase + ch * 16) = w;
+                *(v4i *)(p.htq + token_axis_offset(t.n0 + col, pbase, ch)) = w;
             }
         }
         if (o_tid < N_PER_TILE && t.n0 + o_tid < p.N) {
@@ -737,7 +745,7 @@ struct GroupedProblem {
                 const bool part_ok = t.row0 + (ch >> 3) * 128 < t.end;
                 if (hcol < H && part_ok) {
                     const v4i w = *(const v4i *)(codes + col * S::BM + (((ch ^ (col >> 2)) & (CH - 1)) << 4));
-                    *(v4i *)(p.htq + (int64_t)(half * H + hcol) * p.ldhtq + pbase + ch * 16) = w;
+                    *(v4i *)(p.htq + token_axis_offset(half * H + hcol, pbase, ch)) = w;
                 }
             }
             if (o_tid < S::BN / 2) {
@@ -890,6 +898,9 @@ __global__ __launch_bounds__(256) void grouped_generic_kernel(GroupedArgs p) {
 struct WgradArgs {
     const uint8_t *aq, *as, *bq, *bs;
     int64_t lda, ldas, ldb, ldbs;
+    // Stage-major code matrices (0: row-major): the 128 positions of K stage kt of every row lie together, stage kt at
+    // kt * a_ks, row r of it at r * 128 (lda is 128 then), so a tile's stage is one contiguous run; b_ks likewise.
+    int64_t a_ks, b_ks;
     void *dw;
     int64_t stride_dwe, lddw;
     const int32_t *offsets;
@@ -1070,6 +1081,8 @@ struct WgradProblem {
         c.kt0 = t.kt0;
         c.kt1 = t.kt1;
         c.tail_kt = -1, c.tail_bytes = 0;  // K % 128 == 0 is a precondition of these kernels
+        c.a_ks = p.a_ks ? p.a_ks : 128;
+        c.b_ks = p.b_ks ? p.b_ks : 128;
         const int mrem = p.N - t.m0, nrem = p.Kout - t.n0;
 #pragma unroll
         for (int q = 0; q < S::QA; q++) {
@@ -1349,11 +1362,13 @@ extern "C" int mx_experts_gemm1(const uint8_t *xq, const uint8_t *xs, int64_t T,
         (pre && ldpre < 2 * H) || (htq != nullptr) != (hts != nullptr))
         return MX_EINVAL;
     const int64_t mpad = ((M + 127) / 128 + E) * 128;
-    if (htq && (ldhtq < mpad - 128 * E || ldhts < (mpad - 128 * E) / MX_BLOCK)) return MX_EINVAL;
+    // a leading dimension of exactly 128 on a wider padded axis: htq stage-major, (Mpad/128, H, 128)
+    const bool t_panels = htq && ldhtq == 128 && mpad > 128;
+    if (htq && ((ldhtq < mpad - 128 * E && !t_panels) || ldhts < (mpad - 128 * E) / MX_BLOCK)) return MX_EINVAL;
     if (M == 0 || H == 0) return MX_OK;
     GroupedArgs a = base_args(xq, xs, ldx, ldxs, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
     a.hq = hq, a.ldhq = ldhq, a.hs = hs, a.ldhs = ldhs, a.pre = pre, a.ldpre = ldpre;
-    a.htq = htq, a.ldhtq = ldhtq, a.hts = hts, a.ldhts = ldhts;
+    a.htq = htq, a.ldhtq = ldhtq, a.hts = hts, a.ldhts = ldhts, a.htq_ks = t_panels ? H * 128 : 0;
     if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || (pre && (!aligned(pre, 8) || ldpre % 4)) ||
         (htq && (!aligned(htq, 16) || ldhtq % 16 || !aligned(hts, 4) || ldhts % 4)))
         return MX_EUNSUPPORTED;
@@ -1392,14 +1407,16 @@ extern "C" int mx_experts_gemm2_dgrad(const uint8_t *dq, const uint8_t *ds, int6
         return MX_EINVAL;
     if (gate_dtype != MX_FP32 && gate_dtype != act_dtype) return MX_EINVAL;
     const int64_t mpad = ((M + 127) / 128 + E) * 128;
-    if (ptq && (ldptq < mpad - 128 * E || ldpts < (mpad - 128 * E) / MX_BLOCK)) return MX_EINVAL;
+    // a leading dimension of exactly 128 on a wider padded axis: ptq stage-major, (Mpad/128, 2H, 128)
+    const bool t_panels = ptq && ldptq == 128 && mpad > 128;
+    if (ptq && ((ldptq < mpad - 128 * E && !t_panels) || ldpts < (mpad - 128 * E) / MX_BLOCK)) return MX_EINVAL;
     if (M == 0 || H == 0) return MX_OK;
     GroupedArgs a = base_args(dq, ds, lddq, ldds, token_of, wq, ws, stride_we, ldw, stride_wse, ldws, offsets, E, M, H, K);
     a.token_of = token_of, a.order = order, a.gate = gate, a.gate_f32 = gate_dtype == MX_FP32;
     a.hq = (uint8_t *)hq, a.ldhq = ldhq, a.hs = (uint8_t *)hs, a.ldhs = ldhs;
     a.pre = (void *)pre, a.dpre = dpre, a.ldpre = ldpre, a.dpq = dpq, a.lddpq = lddpq, a.dps = dps, a.lddps = lddps;
     a.dgate = dgate;
-    a.htq = ptq, a.ldhtq = ldptq, a.hts = pts, a.ldhts = ldpts;
+    a.htq = ptq, a.ldhtq = ldptq, a.hts = pts, a.ldhts = ldpts, a.htq_ks = t_panels ? 2 * H * 128 : 0;
     if (K == 0 || !tiled_ok(a, T) || !aligned(hq, 8) || ldhq % 8 || !aligned(pre, 16) || (dpre && !aligned(dpre, 16)) ||
         ldpre % 8 || H % 8 || !aligned(dpq, 8) || lddpq % 8 ||
         (ptq && (!aligned(ptq, 16) || ldptq % 16 || !aligned(pts, 4) || ldpts % 4)))
@@ -1477,7 +1494,10 @@ extern "C" int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t
         Kout >= 0x7FFFFFFF || lddw < Kout || workspace_bytes < 0)
         return MX_EINVAL;
     const int64_t mpad = ((M + 127) / 128 + E) * 128;
-    if (lda < mpad || ldb < mpad || ldas < mpad / MX_BLOCK || ldbs < mpad / MX_BLOCK) return MX_EINVAL;
+    // a leading dimension of exactly 128 on the wider padded axis is the stage-major layout (see the header)
+    const bool a_panels = lda == 128 && mpad > 128, b_panels = ldb == 128 && mpad > 128;
+    if ((lda < mpad && !a_panels) || (ldb < mpad && !b_panels) || ldas < mpad / MX_BLOCK || ldbs < mpad / MX_BLOCK)
+        return MX_EINVAL;
     if (N == 0 || Kout == 0) return MX_OK;
     if (!aligned(aq, 16) || !aligned(bq, 16) || lda % 16 || ldb % 16 || !aligned(as, 4) || !aligned(bs, 4) || ldas % 4 ||
         ldbs % 4 || 256 * lda >= ((int64_t)1 << 32) || 256 * ldb >= ((int64_t)1 << 32))
@@ -1486,6 +1506,7 @@ extern "C" int mx_grouped_wgrad_nt(const uint8_t *aq, const uint8_t *as, int64_t
     a.aq = aq, a.as = as, a.bq = bq, a.bs = bs, a.lda = lda, a.ldas = ldas, a.ldb = ldb, a.ldbs = ldbs;
     a.dw = dw, a.stride_dwe = stride_dwe, a.lddw = lddw, a.offsets = offsets, a.E = (int)E, a.N = (int)N,
     a.Kout = (int)Kout, a.KB = (int)(mpad / MX_BLOCK);
+    a.a_ks = a_panels ? N * 128 : 0, a.b_ks = b_panels ? Kout * 128 : 0;
     hipStream_t st = (hipStream_t)stream;
     if (mx::stream_is_capturing(st)) return MX_ECAPTURE;
     switch (dw_dtype) {

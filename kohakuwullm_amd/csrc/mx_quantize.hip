@@ -1260,7 +1260,9 @@ extern "C" int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, i
     if (source != SRC_PLAIN && source != SRC_SWIGLU) return MX_EINVAL;
     const int64_t tiles = (M + QC_TILE - 1) / QC_TILE + E;
     const int64_t mpad = tiles * QC_TILE;
-    if (ldqT < mpad || ldsT < mpad / MX_BLOCK || ldx < (source == SRC_SWIGLU ? 2 * C : C)) return MX_EINVAL;
+    // a leading dimension of exactly 128 on the wider padded axis: qT stage-major, (Mpad/128, C, 128)
+    const bool qt_panels = ldqT == 128 && mpad > 128;
+    if ((ldqT < mpad && !qt_panels) || ldsT < mpad / MX_BLOCK || ldx < (source == SRC_SWIGLU ? 2 * C : C)) return MX_EINVAL;
     if (row_scale && row_scale_dtype != MX_FP32 && row_scale_dtype != dtype) return MX_EINVAL;
     if (dtype != MX_BF16 && dtype != MX_FP16) return MX_EUNSUPPORTED;
     if (C % 8 || !aligned(x, 16) || (ldx * 2) % 16 || !aligned(qT, 16) || ldqT % 16 || tiles > 65535) return MX_EUNSUPPORTED;
@@ -1268,7 +1270,7 @@ extern "C" int mx_quantize_cols_grouped(const void *x, int dtype, int64_t ldx, i
     GroupedQuantArgs a;
     a.x = x, a.ldx = ldx, a.C = (int)C, a.index = index, a.row_scale = row_scale, a.scale_index = scale_index;
     a.scale_f32 = row_scale_dtype == MX_FP32, a.offsets = offsets, a.E = (int)E;
-    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, nullptr, 0, nullptr, 0);
+    QuantTileOut o = tile_out(qT, ldqT, sT, ldsT, nullptr, 0, nullptr, 0, 0, qt_panels ? C * 128 : 0);
     const int ctiles = (int)((C + QC_TILE - 1) / QC_TILE);
     // four column tiles per workgroup while that still leaves every CU several workgroups
     a.span = ctiles >= 4 && (int64_t)tiles * (ctiles / 4) >= 2 * (int64_t)mx::num_cus() ? 4 : 1;

@@ -22,12 +22,16 @@ from kohakuwullm_amd.kernels.mxfp8.grouped import (
     grouped_mxfp8_wgrad,
     padded_rows,
     token_axis_buffers,
+    token_axis_pitch,
     quantize_mx_cols_grouped,
 )
 from kohakuwullm_amd.kernels.mxfp8.quantize import BLOCK_SCALE, quantize_mx, quantize_mx_cols
 
 _FP8 = torch.float8_e4m3fn
 _ACT_DTYPES = (torch.bfloat16, torch.float16)
+# The token-axis operands of the expert WGRADs (h, dpre, gathered x, gate-scaled dout) are written stage-major,
+# (Mpad // 128, rows, 128): a K stage of a WGRAD tile is then one contiguous run instead of 256 rows ~100 KB apart.
+TOKEN_AXIS_STAGE_MAJOR = True
 
 
 def _quantize_stacked(w: torch.Tensor):
@@ -104,7 +108,8 @@ def _w_args(wq, ws):
 def launch_gemm1(xq, xs, token_of, wq, ws, hq, hs, pre, offsets, hidden, dim, act_dtype, htq=None, hts=None) -> None:
     """GEMM1 with its epilogue; ``token_of=None`` reads row m of ``xq`` for sorted row m.
 
-    ``htq``/``hts`` ``(H, Mpad)``/``(H, Mpad//32)``, when given, receive ``h`` quantized along the tokens.
+    ``htq``/``hts`` ``(H, Mpad)``/``(H, Mpad//32)``, when given, receive ``h`` quantized along the tokens
+    (``htq`` may be stage-major, ``(Mpad//128, H, 128)``).
     """
     m = hq.shape[0]
     _lib.invoke(
@@ -113,7 +118,7 @@ def launch_gemm1(xq, xs, token_of, wq, ws, hq, hs, pre, offsets, hidden, dim, ac
         0 if token_of is None else token_of.data_ptr(), *_w_args(wq, ws),
         offsets.data_ptr(), wq.shape[0], hq.data_ptr(), hq.stride(0), hs.data_ptr(), hs.stride(0),
         0 if pre is None else pre.data_ptr(), 0 if pre is None else pre.stride(0),
-        0 if htq is None else htq.data_ptr(), 0 if htq is None else htq.stride(0),
+        0 if htq is None else htq.data_ptr(), 0 if htq is None else token_axis_pitch(htq),
         0 if hts is None else hts.data_ptr(), 0 if hts is None else hts.stride(0),
         _lib.MX_DTYPE[act_dtype], m, hidden, dim,
     )
@@ -188,7 +193,7 @@ def launch_gemm2_dgrad(dq, ds, token_of, order, gate, wq, ws, hq, hs, pre, dpre,
         hq.data_ptr(), hq.stride(0), hs.data_ptr(), hs.stride(0), pre.data_ptr(),
         0 if dpre is None else dpre.data_ptr(), pre.stride(0),
         dpq.data_ptr(), dpq.stride(0), dps.data_ptr(), dps.stride(0),
-        0 if ptq is None else ptq.data_ptr(), 0 if ptq is None else ptq.stride(0),
+        0 if ptq is None else ptq.data_ptr(), 0 if ptq is None else token_axis_pitch(ptq),
         0 if pts is None else pts.data_ptr(), 0 if pts is None else pts.stride(0),
         dgate.data_ptr(), _lib.MX_DTYPE[pre.dtype], m, hidden, dim,
     )
@@ -210,7 +215,7 @@ class _MXFP8Experts(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             # h along the tokens, for dW_out: written by GEMM1's epilogue instead of a pass over `pre`
             mpad = padded_rows(m, packed.in_fwd[0].shape[0])
-            htq, hts = token_axis_buffers(hidden, mpad, x.device)
+            htq, hts = token_axis_buffers(hidden, mpad, x.device, TOKEN_AXIS_STAGE_MAJOR)
         launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hidden, dim, x.dtype, htq, hts)
         # pairs per token when `order` is the pair index token * top_k + slot; 0 = unknown layout
         top_k = gate.numel() // rows if rows and gate.numel() % rows == 0 else 0
@@ -240,7 +245,7 @@ class _MXFP8Experts(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             # dpre along the tokens, for dW_in: written by the epilogue; dpre itself never reaches memory
             mpad = padded_rows(m, packed.in_fwd[0].shape[0])
-            ptq, pts = token_axis_buffers(2 * hidden, mpad, dev)
+            ptq, pts = token_axis_buffers(2 * hidden, mpad, dev, TOKEN_AXIS_STAGE_MAJOR)
         dpre = None if ptq is not None else torch.empty(m, 2 * hidden, device=dev, dtype=dout.dtype)
         launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets,
                            ptq, pts)
@@ -250,11 +255,12 @@ class _MXFP8Experts(torch.autograd.Function):
         dw_in = dw_out = None
         if ctx.needs_input_grad[2]:
             # dW_out[e] = (gate-scaled dout rows of e).T @ h rows of e; h is rebuilt from `pre`
-            dtq, dts = quantize_mx_cols_grouped(dout, offsets, m, index=token_of, row_scale=gate, scale_index=order)
+            dtq, dts = quantize_mx_cols_grouped(dout, offsets, m, index=token_of, row_scale=gate, scale_index=order,
+                                                stage_major=TOKEN_AXIS_STAGE_MAJOR)
             dw_out = grouped_mxfp8_wgrad(dtq, dts, htq, hts, offsets, m, dout.dtype)
         if ctx.needs_input_grad[1]:
             # dW_in[e] = dpre rows of e .T @ x rows of e
-            xtq, xts = quantize_mx_cols_grouped(x, offsets, m, index=token_of)
+            xtq, xts = quantize_mx_cols_grouped(x, offsets, m, index=token_of, stage_major=TOKEN_AXIS_STAGE_MAJOR)
             dw_in = grouped_mxfp8_wgrad(ptq, pts, xtq, xts, offsets, m, dout.dtype)
         return dx, dw_in, dw_out, dgate.to(gate.dtype), None, None, None, None, None
 
@@ -354,8 +360,8 @@ class _GroupedExpertMatmul(torch.autograd.Function):
                                            out=_maybe_zeros(ctx.sentinel, dout.shape[0], k, dout))
             dx = dx_sorted if index is None else torch.zeros_like(x).index_add_(0, index.long(), dx_sorted)
         if ctx.needs_input_grad[1]:
-            dtq, dts = quantize_mx_cols_grouped(dout, offsets, ctx.rows)
-            xtq, xts = quantize_mx_cols_grouped(x, offsets, ctx.rows, index=index)
+            dtq, dts = quantize_mx_cols_grouped(dout, offsets, ctx.rows, stage_major=TOKEN_AXIS_STAGE_MAJOR)
+            xtq, xts = quantize_mx_cols_grouped(x, offsets, ctx.rows, index=index, stage_major=TOKEN_AXIS_STAGE_MAJOR)
             dw = grouped_mxfp8_wgrad(dtq, dts, xtq, xts, offsets, ctx.rows, dout.dtype)
         return dx, dw, None, None, None, None, None, None, None
 

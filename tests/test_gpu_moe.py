@@ -769,3 +769,73 @@ def test_moe_module_reference_defaults(oracle):
     loop = MoEMLP(256, hidden=128, num_experts=4, top_k=2, num_shared=0, dense_fallback=True).to(DEV)
     rep = swap_mxfp8(loop)
     assert rep.blocking and any("dense_fallback" in why for _, why in rep.skipped)
+
+
+@pytest.mark.parametrize("counts,hid", [([200, 0, 56, 300], 160), ([1, 700], 544), ([130] * 5, 256), ([90], 64)])
+def test_token_axis_operands_stage_major_are_the_same_bytes(counts, hid):
+    """Every writer of a token-axis code matrix (the grouped quantizer with its three sources, GEMM1's and GEMM2-dgrad's
+    epilogues) can lay it out stage-major, (Mpad // 128, rows, 128), and the expert WGRAD reads either layout per
+    operand: the panels hold the row-major bytes, nothing is written past the experts' tiles, scales are untouched and
+    dW is bit-identical whichever way each operand is stored."""
+    from kohakuwullm_amd.kernels.mxfp8.grouped import (
+        grouped_mxfp8_wgrad, padded_rows, quantize_mx_cols_grouped, token_axis_buffers)
+    from kohakuwullm_amd.kernels.mxfp8.moe import MXFP8ExpertWeights, launch_gemm1, launch_gemm2_dgrad
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx, rows_of_stage_major
+
+    g = torch.Generator().manual_seed(SEED + 12)
+    e, dim, top_k = len(counts), 256, 1
+    tokens = sum(counts) + 24
+    offsets, order, token_of = (t.to(DEV) for t in _routing(counts, top_k, tokens))
+    m = sum(counts)
+    mpad = padded_rows(m, e)
+    x = torch.randn(tokens, dim, generator=g).bfloat16().to(DEV)
+    dout = torch.randn(tokens, dim, generator=g).bfloat16().to(DEV)
+    gate = (torch.rand(tokens, generator=g) * 0.5 + 0.5).bfloat16().to(DEV)
+    packed = MXFP8ExpertWeights((torch.randn(e, 2 * hid, dim, generator=g) * 0.06).bfloat16().to(DEV),
+                                (torch.randn(e, dim, hid, generator=g) * 0.06).bfloat16().to(DEV))
+    xq, xs = quantize_mx(x)
+    dq, ds = quantize_mx(dout)
+
+    def run(stage_major):
+        z = lambda *shape, dtype=torch.uint8: torch.zeros(*shape, device=DEV, dtype=dtype)  # noqa: E731
+
+        def zeroed(rows):
+            q, s = token_axis_buffers(rows, mpad, DEV, stage_major)
+            q.view(torch.uint8).zero_()
+            s.zero_()
+            return q, s
+
+        hq, hs, pre = z(m, hid, dtype=F8), z(m, hid // 32), z(m, 2 * hid, dtype=torch.bfloat16)
+        htq, hts = zeroed(hid)
+        launch_gemm1(xq, xs, token_of, *packed.in_fwd, hq, hs, pre, offsets, hid, dim, torch.bfloat16, htq, hts)
+        dpre, dpq, dps = z(m, 2 * hid, dtype=torch.bfloat16), z(m, 2 * hid, dtype=F8), z(m, 2 * hid // 32)
+        ptq, pts = zeroed(2 * hid)
+        dgate = z(tokens, dtype=torch.float32)
+        launch_gemm2_dgrad(dq, ds, token_of, order, gate, *packed.out_dgrad, hq, hs, pre, dpre, dpq, dps, dgate, offsets, ptq, pts)
+        dtq, dts = quantize_mx_cols_grouped(dout, offsets, m, index=token_of, row_scale=gate, scale_index=order,
+                                            stage_major=stage_major)
+        xtq, xts = quantize_mx_cols_grouped(x, offsets, m, index=token_of, stage_major=stage_major)
+        rtq, rts = quantize_mx_cols_grouped(pre, offsets, m, swiglu=True, stage_major=stage_major)
+        torch.cuda.synchronize()
+        return {"h": (htq, hts), "dpre": (ptq, pts), "dout": (dtq, dts), "x": (xtq, xts), "h from pre": (rtq, rts)}
+
+    rows, panels = run(False), run(True)
+    valid = torch.zeros(mpad, dtype=torch.bool)
+    pos = 0
+    for c in counts:
+        tiles = -(-c // 128)
+        valid[pos : pos + tiles * 128] = True
+        pos += tiles * 128
+    for name in rows:
+        (rq, rs), (pq, ps) = rows[name], panels[name]
+        assert pq.dim() == 3 and pq.shape == (mpad // 128, rq.shape[0], 128), name
+        flat = rows_of_stage_major(pq).view(torch.uint8).cpu()
+        assert torch.equal(flat[:, valid], rq.view(torch.uint8).cpu()[:, valid]), name
+        assert torch.equal(ps.cpu()[:, valid.view(-1, 32)[:, 0]], rs.cpu()[:, valid.view(-1, 32)[:, 0]]), name
+        if name in ("h", "dpre"):  # these buffers were zeroed: nothing lands past the experts' tiles
+            assert not flat[:, ~valid].any(), name
+    # dW_out = dout^T h and dW_in = dpre^T x with each operand in either layout
+    for a, b in (("dout", "h"), ("dpre", "x")):
+        want = grouped_mxfp8_wgrad(*rows[a], *rows[b], offsets, m)
+        for la, lb in ((panels, panels), (panels, rows), (rows, panels)):
+            assert torch.equal(grouped_mxfp8_wgrad(*la[a], *lb[b], offsets, m), want), (a, b)
