@@ -147,7 +147,8 @@ struct GemmShape {
     static constexpr int SC_A = 4 * PA * 4, SC_B = 4 * PB * 4;  // bytes per super-step
     static constexpr int LDS_BYTES = 2 * (DATA_A + DATA_B + SC_A + SC_B);
     // + the staging area of SCALES_COPY (16 bytes per row of A and B) and the event counter of the A look-ahead
-    static constexpr int LDS_BYTES_AHEAD = LDS_BYTES + 16 * (BM + BN) + 64;
+    static constexpr int LDS_BYTES_STAGED = LDS_BYTES + 16 * (BM + BN);  // SCALES_COPY without the look-ahead
+    static constexpr int LDS_BYTES_AHEAD = LDS_BYTES_STAGED + 64;
     static constexpr bool TWO_ROWS = BM + BN > NTHR;
     static_assert(NT == 8 || NT == 4, "a lane's NT sub-tiles are NT consecutive N: one 16-byte (or 8-byte) store");
     static_assert(WTM % 16 == 0, "a wave's M extent must be a multiple of 16");

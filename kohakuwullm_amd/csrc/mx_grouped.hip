@@ -17,6 +17,8 @@
 //              SwiGLU' from the stored pre; dpre (M,2H) stored and requantized
 //                                                                         experts_bwd.py:29-164
 // The row gather costs nothing: every lane of the copy engine supplies its own global address.
+#include <type_traits>
+
 #include "mx_gemm_core.h"
 
 namespace mx {
@@ -141,12 +143,19 @@ __device__ __forceinline__ float row16_sum(float a) {
 // with 250 empty experts in front of the busy ones that walk cost every workgroup ~100 us per
 // launch.  More experts than the tables hold fall back to the walk.
 #define MX_TABLE_MAX 1024
-struct ExpertTable {
-    int a[MX_TABLE_MAX + 1];
-    int b[MX_TABLE_MAX + 1];
+template <int MAX>
+struct ExpertTableN {
+    static constexpr int CAPACITY = MAX;
+    int a[MAX + 1];
+    int b[MAX + 1];
     int n;
     int longest;  // build_live_table: the K stages of the expert with the most rows
 };
+typedef ExpertTableN<MX_TABLE_MAX> ExpertTable;
+// The expert dW kernel that stages its scale bytes through LDS has 6 KB left for its table (the dynamic part starts
+// on a multiple of 1 KB: 6 KB + the stage buffers, scale planes and staging area are 159 of the CU's 160 KB).
+#define MX_TABLE_MAX_STAGED 760
+typedef ExpertTableN<MX_TABLE_MAX_STAGED> ExpertTableStaged;
 
 // a[e] = row tiles (of `bm` rows) of experts before e, b[e] = 128-row tiles of the padded token
 // axis before e, for e in [0, E]; n = E.
@@ -177,7 +186,8 @@ __device__ __forceinline__ void build_row_tile_table(int *__restrict__ tab_a, in
 
 // a[j] = the j-th expert with rows, b[j] = 128-token K stages of the experts before it; n = how many;
 // b[n] = K stages of all experts.
-__device__ __forceinline__ void build_live_table(ExpertTable &tb, const int32_t *__restrict__ offsets, int E) {
+template <typename TB>
+__device__ __forceinline__ void build_live_table(TB &tb, const int32_t *__restrict__ offsets, int E) {
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
         const uint64_t below = lane ? ~0ull >> (64 - lane) : 0ull;
@@ -927,7 +937,8 @@ struct WgradEven {
     int per_e, groups, q, total;
 };
 
-__device__ __forceinline__ WgradEven wgrad_even_plan(const WgradArgs &p, int workgroups, const ExpertTable &tb) {
+template <typename TB>
+__device__ __forceinline__ WgradEven wgrad_even_plan(const WgradArgs &p, int workgroups, const TB &tb) {
     WgradEven v;
     v.per_e = p.tiles_m * p.tiles_n;
     v.groups = workgroups / v.per_e;  // > 0: the split is only chosen when the tiles leave workgroups idle
@@ -943,7 +954,8 @@ __device__ __forceinline__ int wgrad_unit_of(int b, int g) { return (g & 7) == 0
 // Number of K slices per tile: as many as fill the GPU about twice over, at most 8, and 1 when
 // the tiles of the non-empty experts already fill three quarters of it.  Also counts the
 // non-empty experts.  (With the table, any result above 1 selects the even split.)
-__device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, int &live, const ExpertTable *tb) {
+template <typename TB>
+__device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, int &live, const TB *tb) {
     if (tb) {
         live = tb->n;
     } else {
@@ -967,7 +979,7 @@ __device__ __forceinline__ int wgrad_slices(const WgradArgs &p, int workgroups, 
     return s < 1 ? 1 : (s > 8 ? 8 : s);
 }
 
-template <typename S, int CDT>
+template <typename S, int CDT, typename TB = ExpertTable>
 struct WgradProblem {
     struct Tile {
         int m0, n0, kt0, kt1, expert;
@@ -993,9 +1005,9 @@ struct WgradProblem {
     // (b % 8) * (G / 8) + b / 8: the workgroups of one XCD take consecutive units, i.e. the tiles
     // of one (expert, K slice), which read the same operand panels, share that XCD's L2 (measured:
     // the kernel's fabric reads equal the operand bytes).
-    const ExpertTable *tb;  // the experts with rows, in LDS, or nullptr (more experts than it holds)
+    const TB *tb;  // the experts with rows, in LDS, or nullptr (more experts than it holds)
 
-    __device__ WgradProblem(const WgradArgs &a, const ExpertTable *table)
+    __device__ WgradProblem(const WgradArgs &a, const TB *table)
         : p(a), kb_end(a.KB), scan_e(0), scan_tiles(0), scan_live(0), tb(table) {
         const int g = (int)gridDim.x, b = (int)blockIdx.x;
         next_unit = wgrad_unit_of(b, g);
@@ -1102,6 +1114,9 @@ struct WgradProblem {
         };
         c.srow0 = srow(L.tid < S::BM + S::BN ? L.tid : 0);
         c.srow1 = S::TWO_ROWS ? srow(L.tid + S::NTHR < S::BM + S::BN ? L.tid + S::NTHR : 0) : nullptr;
+        // SCALES_COPY: the same row through the copy engine, as a 32-bit offset from its matrix
+        c.sa_base = p.as, c.sb_base = p.bs;
+        c.s_voff = (uint32_t)(c.srow0 - (L.tid < S::BM ? p.as : p.bs));
     }
 
     __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
@@ -1163,10 +1178,12 @@ __global__ __launch_bounds__(256) void wgrad_zero_kernel(WgradArgs p, int chunks
 template <typename S, int CDT, int SCALES>
 __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    __shared__ ExpertTable table;
-    const bool tabled = args.E <= MX_TABLE_MAX;
+    // SCALES_COPY (the host selects it only for E <= MX_TABLE_MAX_STAGED): the smaller table beside the staging area
+    typedef typename std::conditional<SCALES == SCALES_COPY, ExpertTableStaged, ExpertTable>::type TB;
+    __shared__ TB table;
+    const bool tabled = args.E <= TB::CAPACITY;
     if (tabled) build_live_table(table, args.offsets, args.E);
-    WgradProblem<S, CDT> prob(args, tabled ? &table : nullptr);
+    WgradProblem<S, CDT, TB> prob(args, tabled ? &table : nullptr);
     persistent_gemm<S, SCALES>(prob, smem);
 }
 
@@ -1472,13 +1489,19 @@ static int launch_wgrad(WgradArgs a, float *ws, int64_t ws_bytes, hipStream_t st
     a.ws = work < (1 << 27) && fits ? ws : nullptr;  // two fp32 tile slots per workgroup, or whole tiles only
     a.slots = a.ws ? 2 * cus : 0;
     dim3 grid((unsigned)(work * (a.slots ? 8 : 1) < cus ? work * (a.slots ? 8 : 1) : cus)), block(S::NTHR);
-    // scale rows with 12 readable bytes behind their last stage take one 16-byte fetch per four stages
+    // scale rows with 12 readable bytes behind their last stage take one 16-byte fetch per four stages ...
     const bool quad = a.ldas >= a.KB + 12 && a.ldbs >= a.KB + 12;
+    // ... and that fetch goes through the copy engine into an LDS staging area (no vector load in the K loop for
+    // the compiler to put a full wait in front of: 10 us of 155 on six experts of 16384 rows) when the lane
+    // offsets fit 32 bits and the experts fit the smaller table that leaves room for the staging area
+    const bool staged = quad && a.E <= MX_TABLE_MAX_STAGED && (int64_t)a.N * a.ldas < ((int64_t)1 << 32) &&
+                        (int64_t)a.Kout * a.ldbs < ((int64_t)1 << 32);
     const int chunks = (a.N + 63) / 64;
     if ((int64_t)a.E * chunks >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
     wgrad_zero_kernel<CDT><<<dim3((unsigned)(a.E * chunks)), dim3(256), 0, st>>>(a, chunks);
-    const int rc = quad ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_QUAD>>(grid, block, S::LDS_BYTES, st, a)
-                        : launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
+    const int rc = staged ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_COPY>>(grid, block, S::LDS_BYTES_STAGED, st, a)
+                   : quad ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_QUAD>>(grid, block, S::LDS_BYTES, st, a)
+                          : launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
     if (rc != MX_OK) return rc;
     // tiles are only split while (tiles x slices) fit the 2 * cus slots, so 4 * cus workgroups cover every unit at once
     const int64_t units = work * S::MT < 4 * (int64_t)cus ? work * S::MT : 4 * (int64_t)cus;
