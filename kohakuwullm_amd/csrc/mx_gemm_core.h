@@ -34,6 +34,7 @@
 #pragma once
 
 #include <atomic>
+#include <type_traits>
 #include <utility>
 
 #include "mx_common.h"
@@ -509,6 +510,15 @@ struct LdsScratch {
 // at least two stages (the caller's guarantee), and the epilogue may not use the stage buffer as scratch (no EARLY_WAIT
 // policy does both).  Same products bit for bit: the MFMA sequence does not change.  Measured inside the feed-forward
 // step: the batched launch of the three long contractions 457 -> 429 us, the K = 1536 products 1 % faster.
+//
+// Under AHEAD a tile's context is built twice, for the A rows one stage before it is built for everything else.  A policy
+// whose context() reads memory (gathered rows) declares `static constexpr bool REUSE_CONTEXT = true` and the second
+// one is a copy of the first.
+template <typename P, typename = void>
+struct reuse_context_of : std::false_type {};
+template <typename P>
+struct reuse_context_of<P, std::void_t<decltype(P::REUSE_CONTEXT)>> : std::integral_constant<bool, P::REUSE_CONTEXT> {};
+
 template <typename S, int K512, typename P, bool AHEAD = false>  // K512: one of SCALES_*
 __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
     static_assert(!(AHEAD && P::EARLY_WAIT), "an epilogue that borrows the stage buffer cannot share it with the look-ahead");
@@ -615,7 +625,8 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
                     }                                                                                         \
                 }                                                                                             \
             } else if (has_next) {                                                                            \
-                prob.context(nxt, L, ctx);                                                                    \
+                if (AHEAD && reuse_context_of<P>::value) ctx = ctxa; /* the next tile's, one stage old */     \
+                else prob.context(nxt, L, ctx);                                                               \
                 if constexpr (COPY) {                                                                         \
                     issue_scales<S>(ctx, L, ctx.kt0 * 4, rawS);                                               \
                 } else {                                                                                      \

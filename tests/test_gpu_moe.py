@@ -49,6 +49,9 @@ COUNT_CASES = [
     # many experts, most of them empty, the busy ones behind long runs of empties: the owner of a
     # tile is found through the per-workgroup expert tables (more than one 64-expert chunk)
     [0] * 70 + [200] + [0] * 130 + [129, 1] + [0] * 50,
+    # more experts than the expert dW kernel's smaller table beside its scale staging area holds (760), fewer than
+    # the full table (1024): the dW kernel with scale bytes in registers
+    [0] * 780 + [150, 40] + [0] * 20,
     # more experts than the tables hold: the kernels fall back to walking `offsets`
     [0] * 1040 + [90, 0, 33] + [0] * 20,
 ]
@@ -82,6 +85,39 @@ def test_grouped_gemm(oracle, counts, use_index):
     # fp32 output: nothing but the MFMA's internal adder between us and fp64
     got32 = grouped_mxfp8_gemm(*_dev(xq, xs), *_dev(wq, ws), offsets.to(DEV), None if index is None else index.to(DEV),
                                out_dtype=torch.float32, rows=m)
+    assert oracle.rel_error(got32.cpu(), ref) < 1e-4
+
+
+@pytest.mark.parametrize("k", [512, 1024])
+@pytest.mark.parametrize("use_index", [False, True])
+def test_grouped_gemm_look_ahead_schedule(oracle, k, use_index):
+    """K a multiple of 512 with 16-byte aligned scale rows takes the schedule that fetches the A operand two K stages
+    ahead and its scale bytes through the copy engine.  More tiles than workgroups, so every workgroup crosses tile
+    boundaries (ragged last tiles, an empty and a one-row expert among them); with and without gathered rows.  Against
+    the fp64 oracle, and bit for bit against the one-stage schedule, which scale rows of another pitch select."""
+    from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_gemm
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator().manual_seed(SEED + 21)
+    counts = [3000, 0, 2500, 1, 4100, 700]
+    e, n, m = len(counts), 1792, sum(counts)  # 43 row tiles x 7 column tiles
+    tokens = 3000 if use_index else m
+    x = torch.randn(tokens, k, generator=g).bfloat16()
+    w = (torch.randn(e * n, k, generator=g) * 0.05).bfloat16()
+    xq, xs = quantize_mx(x.to(DEV))
+    wq, ws = quantize_mx(w.to(DEV))
+    wq, ws = wq.view(e, n, k), ws.view(e, n, k // 32)
+    offsets = torch.zeros(e + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    index = torch.randint(0, tokens, (m,), generator=g).int().to(DEV) if use_index else None
+    got = grouped_mxfp8_gemm(xq, xs, wq, ws, offsets.to(DEV), index, rows=m)
+    ref = oracle.grouped_gemm_nt(xq.view(torch.uint8).cpu(), xs.cpu(), wq.view(torch.uint8).cpu(), ws.cpu(), offsets,
+                                 None if index is None else index.cpu())
+    assert oracle.rel_error(got.cpu(), ref) < TOL
+    xs_other = torch.empty(tokens, k // 32 + 4, device=DEV, dtype=torch.uint8)[:, : k // 32]  # pitch not a multiple of 16
+    xs_other.copy_(xs)
+    assert torch.equal(got, grouped_mxfp8_gemm(xq, xs_other, wq, ws, offsets.to(DEV), index, rows=m))
+    got32 = grouped_mxfp8_gemm(xq, xs, wq, ws, offsets.to(DEV), index, out_dtype=torch.float32, rows=m)
     assert oracle.rel_error(got32.cpu(), ref) < 1e-4
 
 
