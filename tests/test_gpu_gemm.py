@@ -332,6 +332,32 @@ def test_gemm_random_shapes(oracle):
         assert oracle.rel_error(out.cpu(), ref) < TOL_BF16, tuple(dev[0].shape)
 
 
+@pytest.mark.parametrize("m,n,k", [(4500, 4200, 2048), (2100, 9000, 1024), (7000, 2300, 1536), (3000, 3000, 3072), (300, 70000, 1024)])
+def test_gemm_look_ahead_schedule_many_tiles(m, n, k):
+    """K % 512 == 0 with 16-byte aligned scale rows takes the schedule that fetches the A operand two K stages ahead and
+    its scale bytes through the copy engine.  More tiles than workgroups (every workgroup crosses tile boundaries, the
+    last round is K-split), ragged edges.  Bit for bit against the one-stage schedule, which scale rows of another
+    pitch select and which the oracle tests of this file pin; and, so that the comparison cannot be of two equal
+    mistakes, against torch's fp32 product of the dequantized operands on the device."""
+    from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
+
+    g = torch.Generator(device=DEV).manual_seed(SEED + k + m)
+    a = torch.randn(m, k, generator=g, device=DEV, dtype=torch.bfloat16)
+    b = torch.randn(n, k, generator=g, device=DEV, dtype=torch.bfloat16) * 0.02
+    aq, as_ = quantize_mx(a)
+    bq, bs = quantize_mx(b)
+    got = _mx().mxfp8_matmul_pq(aq, as_, bq, bs, torch.float32)
+    as_other = torch.empty(m, k // 32 + 4, device=DEV, dtype=torch.uint8)[:, : k // 32]  # pitch not a multiple of 16
+    as_other.copy_(as_)
+    assert torch.equal(got, _mx().mxfp8_matmul_pq(aq, as_other, bq, bs, torch.float32))
+    deq = lambda q, sc: q.float() * torch.exp2(sc.float() - 127.0).repeat_interleave(32, dim=1)  # noqa: E731
+    ref = deq(aq, as_) @ deq(bq, bs).T
+    assert float((got - ref).norm() / ref.norm()) < TOL_FP32
+    got16 = _mx().mxfp8_matmul_pq(aq, as_, bq, bs, torch.bfloat16)
+    assert torch.equal(got16, _mx().mxfp8_matmul_pq(aq, as_other, bq, bs, torch.bfloat16))
+    assert torch.equal(got16, got.bfloat16())
+
+
 def test_gemm_split_on_two_streams(oracle):
     """Launches that use the K-split scratch on different streams at the same time do not share it."""
     m, n, k = 512, 512, 8192  # 4 tiles, long K: the even split
