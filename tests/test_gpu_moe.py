@@ -90,18 +90,19 @@ def test_grouped_gemm(oracle, counts, use_index):
 
 @pytest.mark.parametrize("k", [512, 1024])
 @pytest.mark.parametrize("use_index", [False, True])
-def test_grouped_gemm_look_ahead_schedule(oracle, k, use_index):
+@pytest.mark.parametrize("counts,n", [([3000, 0, 2500, 1, 4100, 700], 1792), ([5, 0, 130], 264), ([0, 0, 1], 8), ([257] * 9, 512)])
+def test_grouped_gemm_look_ahead_schedule(oracle, k, use_index, counts, n):
     """K a multiple of 512 with 16-byte aligned scale rows takes the schedule that fetches the A operand two K stages
     ahead and its scale bytes through the copy engine.  More tiles than workgroups, so every workgroup crosses tile
-    boundaries (ragged last tiles, an empty and a one-row expert among them); with and without gathered rows.  Against
+    boundaries (ragged last tiles, an empty and a one-row expert among them), and launches of one or a few tiles; with
+    and without gathered rows.  Against
     the fp64 oracle, and bit for bit against the one-stage schedule, which scale rows of another pitch select."""
     from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_gemm
     from kohakuwullm_amd.kernels.mxfp8.quantize import quantize_mx
 
     g = torch.Generator().manual_seed(SEED + 21)
-    counts = [3000, 0, 2500, 1, 4100, 700]
-    e, n, m = len(counts), 1792, sum(counts)  # 43 row tiles x 7 column tiles
-    tokens = 3000 if use_index else m
+    e, m = len(counts), sum(counts)  # the first case: 43 row tiles x 7 column tiles; the others: at most a tile per workgroup
+    tokens = max(m // 3, 8) if use_index else m
     x = torch.randn(tokens, k, generator=g).bfloat16()
     w = (torch.randn(e * n, k, generator=g) * 0.05).bfloat16()
     xq, xs = quantize_mx(x.to(DEV))
