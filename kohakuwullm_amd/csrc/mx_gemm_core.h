@@ -80,6 +80,23 @@ __device__ __forceinline__ void dma16_run2(const uint8_t *biased_base, uint32_t 
                  : "memory");
 }
 
+// The same run with both halves of the execution mask set to `mask` around it (all ones, or zero: the copies are issued
+// and move nothing).  A wave-uniform "whether", without a branch in the stage body.
+template <int P0>
+__device__ __forceinline__ void dma16_run2_masked(const uint8_t *biased_base, uint32_t v0, uint32_t v1, uint32_t lds, uint32_t mask) {
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\t"
+                 "s_mov_b32 exec_lo, %5\n\t"
+                 "s_mov_b32 exec_hi, %5\n\t"
+                 "s_mov_b32 m0, %4\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %3 offset:%6\n\t"
+                 "global_load_lds_dwordx4 %2, %3 offset:%7\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "v"(v0), "v"(v1), "s"(biased_base), "s"(lds), "s"(mask), "n"(P0 * 1024), "n"((P0 + 1) * 1024)
+                 : "memory");
+}
+
 __device__ __forceinline__ void dma16_run4(const uint8_t *biased_base, uint32_t v0, uint32_t v1, uint32_t v2, uint32_t v3,
                                            uint32_t lds) {
     asm volatile("s_mov_b32 m0, %5\n\ts_nop 0\n\t"
@@ -264,15 +281,19 @@ struct CopyRuns {
     static constexpr int RUN = MX_COPY_RUN;
     static_assert(S::QA % RUN == 0 && S::QB % RUN == 0 && COPY_GROUP % RUN == 0, "whole runs inside a group of four");
     static constexpr int RA = S::QA / RUN, RB = S::QB / RUN, N = RA + RB;
-    template <int R>
+    template <int R, bool MASKED = false>
     static __device__ __forceinline__ void issue(const IssueCtx<S> &c, const Lane &L, int kt, const uint8_t *ga,
-                                                 const uint8_t *gb, uint32_t wa, uint32_t wb) {
+                                                 const uint8_t *gb, uint32_t wa, uint32_t wb, uint32_t mask = ~0u) {
         constexpr bool B = R >= RA;
         constexpr int q0 = (B ? R - RA : R) * RUN;
         const uint8_t *g = B ? gb : ga;
         const uint32_t lds = (B ? wb : wa) + (q0 / COPY_GROUP) * (COPY_GROUP * 1024);
         const uint32_t *voff = B ? c.b_voff : c.a_voff;
-        if constexpr (RUN == 2)
+        static_assert(!MASKED || RUN == 2, "masked copies come in runs of two");
+        if constexpr (MASKED)
+            dma16_run2_masked<q0 % COPY_GROUP>(g, voff[q0] - tail_fix<S>(c, L, kt, q0), voff[q0 + 1] - tail_fix<S>(c, L, kt, q0 + 1), lds,
+                                               mask);
+        else if constexpr (RUN == 2)
             dma16_run2<q0 % COPY_GROUP>(g, voff[q0] - tail_fix<S>(c, L, kt, q0), voff[q0 + 1] - tail_fix<S>(c, L, kt, q0 + 1), lds);
         else
             dma16_run4(g, voff[q0] - tail_fix<S>(c, L, kt, q0), voff[q0 + 1] - tail_fix<S>(c, L, kt, q0 + 1),
@@ -286,6 +307,21 @@ struct CopyRuns {
 __device__ __forceinline__ Lane opaque(const Lane &L) {
     Lane R = L;
     asm volatile("" : "+v"(R.tid), "+v"(R.lane));
+    return R;
+}
+
+// The whole descriptor rebuilt from such a copy: for an epilogue whose per-lane addresses would otherwise be invariants of
+// the tile loop, computed once in front of it and spilled across the K loop.  (A spill in front of the loop costs more
+// than its two instructions: every write inside the loop to a register the pending scratch store reads gets a full
+// vector-memory wait in front of it, which also waits for the stage's copies.)
+template <typename S>
+__device__ __forceinline__ Lane rebuilt(const Lane &L) {
+    Lane R = opaque(L);
+    R.wave = __builtin_amdgcn_readfirstlane(R.tid >> 6);
+    R.wm = R.wave / S::WGN;
+    R.wn = R.wave % S::WGN;
+    R.r16 = R.lane & 15;
+    R.g = R.lane >> 4;
     return R;
 }
 
@@ -398,14 +434,15 @@ __device__ __forceinline__ void park_staged(const Lane &L, const uint8_t *raw, u
 // AHEAD (the A look-ahead, see persistent_gemm): the stage fetches the B rows of stage `kt_next` into buffer `buf_next`
 // in its first steps and, in steps 4 and 5, the A rows of stage `kt_a` of the tile `ca` describes -- the stage after
 // `kt_next` in the workgroup's sequence of stages -- into the A half of the buffer it is itself reading, once every wave
-// has its A fragments of this stage in registers (`counter` has reached `target`).
-template <typename S, int OPSEL, bool AHEAD = false>
+// has its A fragments of this stage in registers (`counter` has reached `target`).  MASKED_A: `a_exec` is the execution
+// mask of those A copies, zero when the stage two on is not known yet (persistent_gemm, tiles of one stage).
+template <typename S, int OPSEL, bool AHEAD = false, bool MASKED_A = false>
 __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, const uint8_t *__restrict__ lb, int a_lo,
                                               int a_hi, int b_lo, int b_hi, const int (&sa)[S::MT],
                                               const int (&sb)[S::NT], v4f (&acc)[S::MT][S::NT],
                                               const IssueCtx<S> &c, const Lane &L, int kt_next, uint8_t *ldsA,
                                               uint8_t *ldsB, int buf_next, const IssueCtx<S> &ca, int kt_a,
-                                              uint32_t counter, uint32_t target) {
+                                              uint32_t counter, uint32_t target, uint32_t a_exec = ~0u) {
     const uint8_t *ga = uniform_ptr((AHEAD ? ca.a_base + (int64_t)kt_a * ca.a_ks : c.a_base + (int64_t)kt_next * c.a_ks) - COPY_BIAS);
     const uint8_t *gb = uniform_ptr(c.b_base + (int64_t)kt_next * c.b_ks - COPY_BIAS);
     const uint32_t wa =
@@ -449,7 +486,7 @@ __device__ __forceinline__ void compute_stage(const uint8_t *__restrict__ la, co
             if constexpr (AHEAD) {
                 constexpr bool isb = r.value >= Runs::RA;
                 if constexpr (isb && r.value - Runs::RA == j) Runs::template issue<r.value>(c, L, kt_next, ga, gb, wa, wb);
-                if constexpr (!isb && A_STEP + r.value == j) Runs::template issue<r.value>(ca, L, kt_a, ga, gb, wa, wb);
+                if constexpr (!isb && A_STEP + r.value == j) Runs::template issue<r.value, MASKED_A>(ca, L, kt_a, ga, gb, wa, wb, a_exec);
             } else if constexpr (r.value * STEPS / Runs::N == j && j < STEPS) {
                 Runs::template issue<r.value>(c, L, kt_next, ga, gb, wa, wb);
             }
@@ -507,8 +544,8 @@ struct LdsScratch {
 // -- and B one stage ahead as before.  The stage-ending wait then leaves the wave's youngest S::QA copies, those A rows,
 // in flight: they have another whole stage to land.  Stages are numbered through the workgroup's whole sequence of
 // tiles, so the last two stages of a tile fetch the A rows of the next tile's first two; every tile must therefore have
-// at least two stages (the caller's guarantee), and the epilogue may not use the stage buffer as scratch (no EARLY_WAIT
-// policy does both).  Same products bit for bit: the MFMA sequence does not change.  Measured inside the feed-forward
+// at least two stages (the caller's guarantee, or the policy declares SHORT_TILES, below), and the epilogue may not use
+// the stage buffer as scratch (no EARLY_WAIT policy does both).  Same products bit for bit: the MFMA sequence does not change.  Measured inside the feed-forward
 // step: the batched launch of the three long contractions 457 -> 429 us, the K = 1536 products 1 % faster.
 //
 // Under AHEAD a tile's context is built twice, for the A rows one stage before it is built for everything else.  A policy
@@ -519,8 +556,20 @@ struct reuse_context_of : std::false_type {};
 template <typename P>
 struct reuse_context_of<P, std::void_t<decltype(P::REUSE_CONTEXT)>> : std::integral_constant<bool, P::REUSE_CONTEXT> {};
 
+//
+// Tiles of a single stage under AHEAD (a policy with `static constexpr bool SHORT_TILES = true`; the others keep the
+// two-stage guarantee).  The stage two on then lies in the tile after the next, which is not known yet: the stage
+// issues no A copies (masked out) and closes with a full wait, and the stage after it fetches its successor's A rows
+// together with the B rows, one stage ahead, before it goes on looking two ahead.
+template <typename P, typename = void>
+struct short_tiles_of : std::false_type {};
+template <typename P>
+struct short_tiles_of<P, std::void_t<decltype(P::SHORT_TILES)>> : std::integral_constant<bool, P::SHORT_TILES> {};
+
 template <typename S, int K512, typename P, bool AHEAD = false>  // K512: one of SCALES_*
 __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
+    constexpr bool SHORT = AHEAD && short_tiles_of<P>::value;
+    bool pend = false;  // SHORT: the A rows of the next stage are not in flight yet; this stage fetches them first
     static_assert(!(AHEAD && P::EARLY_WAIT), "an epilogue that borrows the stage buffer cannot share it with the look-ahead");
     uint8_t *const ldsA = smem;                                                  // [2][BM*128]
     uint8_t *const ldsB = smem + 2 * S::DATA_A;                                  // [2][BN*128]
@@ -564,7 +613,8 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
         }
         issue_stage<S>(ctx, L, ctx.kt0, ldsA, ldsB, 0);
         if (AHEAD) {
-            issue_a<S>(ctx, L, ctx.kt0 + 1, ldsA, 1);
+            if (!SHORT || ctx.kt1 - ctx.kt0 >= 2) issue_a<S>(ctx, L, ctx.kt0 + 1, ldsA, 1);
+            else pend = true;
             if (L.tid == 0) *(volatile uint32_t *)(smem + S::LDS_BYTES + 16 * (S::BM + S::BN)) = 0;
         }
         if constexpr (!COPY) {
@@ -640,19 +690,28 @@ __device__ __forceinline__ void persistent_gemm(P &prob, uint8_t *smem) {
             /* AHEAD: the A rows two stages on: this tile's, or the next tile's first two (its context  */    \
             /* from the second-to-last stage on), or, with no tile left, a re-read nobody will look at. */    \
             int kt_a = kt0 + k + 2;                                                                           \
+            bool known = true; /* SHORT: whether the stage two on is in this tile or the next */              \
             if (AHEAD && k + 2 >= KT) {                                                                       \
                 if (has_next) {                                                                               \
-                    if (k + 2 == KT) prob.context(nxt, L, ctxa);                                              \
+                    if (SHORT ? k == (KT >= 2 ? KT - 2 : 0) : k + 2 == KT) prob.context(nxt, L, ctxa);        \
                     kt_a = ctxa.kt0 + (k + 2 - KT);                                                           \
+                    if (SHORT) known = k + 2 - KT < ctxa.kt1 - ctxa.kt0;                                      \
                 } else {                                                                                      \
                     kt_a = kt0 + k;                                                                           \
                 }                                                                                             \
             }                                                                                                 \
-            compute_stage<S, SIDX, AHEAD>(ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64,    \
-                                          b_rd, b_rd ^ 64, sa, sb, acc, ctx, L, kt_issue, ldsA, ldsB,         \
-                                          buf ^ 1, ctxa, kt_a, counter, (uint32_t)(gstage + 1) * S::NW);      \
+            if constexpr (SHORT) {                                                                            \
+                /* the next stage's A rows, which no earlier stage could fetch: with its B rows, up front */  \
+                if (pend) issue_a<S>(ctx, L, kt_issue, ldsA, buf ^ 1);                                        \
+                pend = !known;                                                                                \
+            }                                                                                                 \
+            compute_stage<S, SIDX, AHEAD, SHORT>(                                                             \
+                ldsA + buf * S::DATA_A, ldsB + buf * S::DATA_B, a_rd, a_rd ^ 64, b_rd, b_rd ^ 64, sa, sb,     \
+                acc, ctx, L, kt_issue, ldsA, ldsB, buf ^ 1, ctxa, kt_a, counter,                              \
+                (uint32_t)(gstage + 1) * S::NW, __builtin_amdgcn_readfirstlane(known ? ~0u : 0u));            \
             if (!last) {                                                                                      \
-                wait_vm_allow_c<AHEAD ? S::QA : 0>();                                                         \
+                if (SHORT && !known) wait_vm_allow_c<0>();                                                    \
+                else wait_vm_allow_c<AHEAD ? S::QA : 0>();                                                    \
                 __syncthreads();                                                                              \
             }                                                                                                 \
             gstage++;                                                                                         \

@@ -1006,6 +1006,8 @@ struct WgradProblem {
     WgradEven ev;
     static constexpr int NST = S::MT * 4 * (CDT == MX_FP32 ? 2 : 1);
     static constexpr bool EARLY_WAIT = false;
+    // an expert of up to 128 rows is one K stage, and so is the end of a range of the even split: see persistent_gemm
+    static constexpr bool SHORT_TILES = true;
 
     // Workgroups are dealt to the 8 XCDs round-robin, so workgroup b starts at unit
     // (b % 8) * (G / 8) + b / 8: the workgroups of one XCD take consecutive units, i.e. the tiles
@@ -1125,7 +1127,8 @@ struct WgradProblem {
         c.s_voff = (uint32_t)(c.srow0 - (L.tid < S::BM ? p.as : p.bs));
     }
 
-    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
+    __device__ __forceinline__ int epilogue(const Tile &t, const Lane &L0, v4f (&acc)[S::MT][S::NT], const LdsScratch &) const {
+        const Lane L = rebuilt<S>(L0);  // no per-lane address of the epilogue lives across the K loop
         if (t.slot >= 0) {  // one K slice: fp32 partial, laid out [sub-tile][thread]
             v4f *dst = (v4f *)p.ws + (int64_t)t.slot * (S::BM * S::BN / 4);
 #pragma unroll
@@ -1190,7 +1193,8 @@ __global__ __launch_bounds__(S::NTHR) void grouped_wgrad_kernel(WgradArgs args) 
     const bool tabled = args.E <= TB::CAPACITY;
     if (tabled) build_live_table(table, args.offsets, args.E);
     WgradProblem<S, CDT, TB> prob(args, tabled ? &table : nullptr);
-    persistent_gemm<S, SCALES>(prob, smem);
+    // with the staged scale bytes goes the A look-ahead of the dense kernels (its K loop then holds no vector load)
+    persistent_gemm<S, SCALES, WgradProblem<S, CDT, TB>, SCALES == SCALES_COPY>(prob, smem);
 }
 
 // Adds the K slices of every tile of every non-empty expert, in slice order, and stores dW.
@@ -1518,7 +1522,7 @@ static int launch_wgrad(WgradArgs a, float *ws, int64_t ws_bytes, hipStream_t st
     const int chunks = (a.N + 63) / 64;
     if ((int64_t)a.E * chunks >= 0x7FFFFFFF) return MX_EUNSUPPORTED;
     wgrad_zero_kernel<CDT><<<dim3((unsigned)(a.E * chunks)), dim3(256), 0, st>>>(a, chunks);
-    const int rc = staged ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_COPY>>(grid, block, S::LDS_BYTES_STAGED, st, a)
+    const int rc = staged ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_COPY>>(grid, block, S::LDS_BYTES_AHEAD, st, a)
                    : quad ? launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_QUAD>>(grid, block, S::LDS_BYTES, st, a)
                           : launch_with_lds<grouped_wgrad_kernel<S, CDT, SCALES_DWORD>>(grid, block, S::LDS_BYTES, st, a);
     if (rc != MX_OK) return rc;

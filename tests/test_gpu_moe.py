@@ -288,6 +288,39 @@ def test_wgrad_even_k_split_ranges_straddle_experts(oracle, counts):
             assert oracle.rel_error(dw[i].cpu(), ref) < TOL, (i, cnt)
 
 
+@pytest.mark.parametrize("counts,n,k", [([50] * 300, 256, 256), ([50, 300, 1, 129, 128, 5, 0, 257] * 45, 512, 256),
+                                        ([128] * 130 + [4000] + [1] * 140, 256, 512)])
+def test_wgrad_runs_of_single_stage_tiles(oracle, counts, n, k):
+    """More (expert, tile) units than workgroups, most of them a single K stage (experts of up to 128 rows), in runs and
+    mixed with longer ones: the expert dW kernel fetches its A operand two stages ahead, and a stage that lies two tiles
+    on is fetched one stage ahead instead.  Every expert against the fp64 oracle."""
+    from kohakuwullm_amd.kernels.mxfp8.grouped import grouped_mxfp8_wgrad, quantize_mx_cols_grouped
+
+    g = torch.Generator().manual_seed(SEED + 8)
+    e, m = len(counts), sum(counts)
+    offsets = torch.zeros(e + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    a = (torch.randn(m, n, generator=g) * 1e-2).bfloat16()
+    b = torch.randn(m, k, generator=g).bfloat16()
+    atq, ats = quantize_mx_cols_grouped(a.to(DEV), offsets.to(DEV), m, stage_major=True)
+    btq, bts = quantize_mx_cols_grouped(b.to(DEV), offsets.to(DEV), m)
+    dw = grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets.to(DEV), m)
+    assert torch.equal(dw, grouped_mxfp8_wgrad(atq, ats, btq, bts, offsets.to(DEV), m))  # deterministic
+    aq_ref, as_ref, _ = _padded_cols_ref(oracle, a.float(), offsets)
+    bq_ref, bs_ref, _ = _padded_cols_ref(oracle, b.float(), offsets)
+    ad, bd = oracle.dequant(aq_ref, as_ref), oracle.dequant(bq_ref, bs_ref)
+    dw = dw.cpu()
+    pos = 0
+    for i, cnt in enumerate(counts):
+        tiles = -(-cnt // 128)
+        ref = ad[:, pos : pos + tiles * 128] @ bd[:, pos : pos + tiles * 128].T
+        pos += tiles * 128
+        if cnt == 0:
+            assert (dw[i] == 0).all()
+        else:
+            assert oracle.rel_error(dw[i], ref) < TOL, (i, cnt)
+
+
 def _expert_oracle(ora, x, w_in, w_out, gate, token_of, order, offsets, dout):
     """The fused path's arithmetic restated with oracle primitives, stage by stage."""
     e, two_h, dim = w_in.shape
