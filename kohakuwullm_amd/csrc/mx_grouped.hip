@@ -412,8 +412,9 @@ struct GroupedProblem {
     // (The epilogue is bound by its vector ALU work -- rounding, sigmoid, two quantizers per
     // value -- not by its stores: staging the row-direction outputs through LDS for wider
     // stores was measured and did not pay.)
-    __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L, v4f (&acc)[S::MT][S::NT],
+    __device__ __forceinline__ int epilogue_gemm1(const Tile &t, const Lane &L0, v4f (&acc)[S::MT][S::NT],
                                                   const LdsScratch &lds) const {
+        const Lane L = rebuilt<S>(L0);  // no per-lane column or row number of the epilogue lives across the K loop
         static_assert(S::MT % 2 == 0 && N_PER_TILE * S::BM <= S::DATA_A, "token-axis staging: one A half holds the tile");
         static_assert(S::NT == 8 && S::BM % 128 == 0, "four gate and four value sub-tiles per lane; whole 128-token tiles");
         constexpr int CH = S::BM / 16;  // 16-byte chunks of a staged column (its BM tokens)
