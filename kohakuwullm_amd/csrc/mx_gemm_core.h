@@ -313,7 +313,8 @@ __device__ __forceinline__ Lane opaque(const Lane &L) {
 // The whole descriptor rebuilt from such a copy: for an epilogue whose per-lane addresses would otherwise be invariants of
 // the tile loop, computed once in front of it and spilled across the K loop.  (A spill in front of the loop costs more
 // than its two instructions: every write inside the loop to a register the pending scratch store reads gets a full
-// vector-memory wait in front of it, which also waits for the stage's copies.)
+// vector-memory wait in front of it, which also waits for the stage's copies.)  Only for policies that run under
+// lane_of's wave -> sub-tile mapping: a schedule that deals the waves differently hands its epilogue its own descriptor.
 template <typename S>
 __device__ __forceinline__ Lane rebuilt(const Lane &L) {
     Lane R = opaque(L);
